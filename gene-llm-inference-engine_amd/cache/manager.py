@@ -51,7 +51,10 @@ class PageGroup:
         self.storage = None
         self.table_dev = None
         if allocate_storage:
-            self.storage = torch.zeros((len(entries), n_pages + 1, 2, need.n_kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
+            if need.value_dim is None or need.value_dim == need.head_dim:
+                self.storage = torch.zeros((len(entries), n_pages + 1, 2, need.n_kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
+            else:         # keys [kv_head][place][head_dim], then values [kv_head][value_dim][place]: a page is one run of numbers
+                self.storage = torch.zeros((len(entries), n_pages + 1, page_size * need.elements_per_position()), dtype=dtype, device=device)
             self.table_dev = torch.tensor(self.table_host, dtype=torch.int32, device=device)
 
     def _changed(self, slot: int, first_entry: int) -> None:
@@ -80,10 +83,11 @@ class PageGroup:
 
     def drop_behind_window(self, slot: int, length: int) -> None:
         """After `length` positions the next row is at position `length`; it sees keys from
-        length - window + 1 on, so pages that end at or before that are given back."""
-        if self.need.window is None:
+        length - window + 1 on (from the start of its chunk on, where the mask is cut into chunks), so pages that end at
+        or before that are given back."""
+        if not self.need.forgets:
             return
-        keep_from = (length - self.need.window + 1) // self.page_size       # first page still visible
+        keep_from = self.need.first_visible(length) // self.page_size       # first page still visible
         first = i = int(self.first_live[slot])
         while i < min(keep_from, int(self.n_held[slot])):
             self.pool.release(int(self.table_host[slot, i]))
@@ -108,9 +112,9 @@ class PageGroup:
 
     def can_rewind_to(self, slot: int, length: int) -> bool:
         """Whether the pages the row at position `length` sees are still held (a window may have given them back)."""
-        if self.need.window is None or length == 0:
+        if not self.need.forgets or length == 0:
             return True
-        return int(self.first_live[slot]) <= max(0, length - self.need.window + 1) // self.page_size
+        return int(self.first_live[slot]) <= self.need.first_visible(length) // self.page_size
 
     def pages_freed_by_rewind(self, slot: int, length: int) -> int:
         first = max(-(-length // self.page_size), int(self.first_live[slot]))
@@ -217,7 +221,7 @@ class CacheManager:
         """Lets requests share the pages of equal prompt prefixes (`self.prefix`).  Possible when pages without a
         window hold all of a request's past, in one group or in several: with a window, pages of a prefix are given
         back while it is still shared; with fixed-size state, the state after the prefix would have to be kept too."""
-        if self.prefix is None and self.groups and all(g.need.window is None for g in self.groups) and not self._state_needed:
+        if self.prefix is None and self.groups and all(not g.need.forgets for g in self.groups) and not self._state_needed:
             self.prefix = PrefixIndex(self.groups[0].pool, self.page_size, [g.pool for g in self.groups[1:]])
         return self.prefix is not None
 
@@ -383,7 +387,7 @@ class CacheManager:
         for r, n in zip(requests, lengths):
             self._length[r] = n + 1
         for g in self.groups:
-            if g.need.window is not None:
+            if g.need.forgets:
                 for slot, n in zip(slots, lengths):
                     g.drop_behind_window(slot, n + 1)
 
@@ -414,7 +418,7 @@ class CacheManager:
             raise CacheError("a request with fixed-size state cannot be rewound: the state of earlier positions is gone")
         for g in self.groups:
             if not g.can_rewind_to(slot, length):
-                raise CacheError(f"request {request!r} cannot be rewound to {length}: a window of {g.need.window} has given those pages back")
+                raise CacheError(f"request {request!r} cannot be rewound to {length}: a window or a chunk's end has given those pages back")
         for g in self.groups:
             if g.shared_page_at(slot, length) and g.pool.free_count + g.pages_freed_by_rewind(slot, length) < 1 and self.evict(1) < 1:
                 raise OutOfPages("no free page to copy a shared page into")

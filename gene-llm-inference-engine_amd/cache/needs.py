@@ -9,13 +9,30 @@ import torch
 
 @dataclass(frozen=True)
 class PagedKvNeed:
-    """Keys and values of every position (or of the last `window` positions) in pages."""
+    """Keys and values of every position (or of the last `window` positions, or of the positions of the chunk of `chunk`
+    positions that the request is in: what no later position can see is given back) in pages.  `value_dim`: channels of a
+    value head where they differ from a key head's `head_dim`."""
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    value_dim: Optional[int] = None
+    chunk: Optional[int] = None
 
     def elements_per_position(self) -> int:
-        return 2 * self.n_kv_heads * self.head_dim
+        return self.n_kv_heads * (self.head_dim + (self.value_dim or self.head_dim))
+
+    def first_visible(self, position: int) -> int:
+        """The earliest position that the row at `position` (and so every later row) may still see."""
+        first = 0
+        if self.window is not None:
+            first = max(first, position - self.window + 1)
+        if self.chunk is not None:
+            first = max(first, position - position % self.chunk)
+        return first
+
+    @property
+    def forgets(self) -> bool:
+        return self.window is not None or self.chunk is not None
 
 
 @dataclass(frozen=True)

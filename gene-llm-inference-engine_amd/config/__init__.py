@@ -1,7 +1,8 @@
 """Typed configurations, the architecture registry and the neutral model description."""
-from .spec import (AttentionSpec, LayerSpec, ModelSpec, RmsNormSpec, RotarySpec,
+from .spec import (AttentionSpec, LayerSpec, MlstmSpec, ModelSpec, PartialRotarySpec, RmsNormSpec, RotarySpec,
                    RunEntry, ScaleSpec, SoftCapSpec, SwiGluSpec)
 from .errors import ConfigError
 from .registry import (config_class_for, parse_config, read_config, register_architecture,
                        registered_architectures)
 from .llama import Llama3Scaling, LlamaConfig          # registers itself
+from .fekorax import FekoraxConfig                     # registers itself

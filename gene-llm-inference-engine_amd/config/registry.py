@@ -1,7 +1,7 @@
 """One registry from an architecture's name to its configuration class.
 
-config.json names its architecture in `architectures[0]` (for instance "LlamaForCausalLM");
-files without that key are matched by `model_type`.  The reference has no registry: one class
+config.json names its architecture in `architectures[0]` (for instance "LlamaForCausalLM") or in
+a string `architecture`; files without either key are matched by `model_type`.  The reference has no registry: one class
 serves its two model types through a flag (src/loader/hf_checkpoint.cpp:96-111).  Here every
 architecture registers a configuration class with `from_dict(dict)` and `model_spec()`, from its
 own module; this one names none of them.
@@ -37,6 +37,8 @@ def config_class_for(cfg: dict) -> type:
     archs = cfg.get("architectures")
     if isinstance(archs, list) and archs:
         name = archs[0]
+    elif isinstance(cfg.get("architecture"), str):           # (files that name one architecture, as a string)
+        name = cfg["architecture"]
     else:
         name = _BY_MODEL_TYPE.get(cfg.get("model_type"))
     if name not in _BY_ARCHITECTURE:

@@ -31,6 +31,23 @@ class RotarySpec:
 
 
 @dataclass(frozen=True)
+class PartialRotarySpec:
+    """Rotation of the pairs (k, k + rotary_dim/2) of the first `rotary_dim` channels of every head by pos * f_k; the other
+    channels of the head pass unchanged.  f_k = theta^(-2k/rotary_dim) unless the architecture gives its own `frequencies`."""
+    kind: ClassVar[str] = "rotary_partial"
+    head_dim: int
+    rotary_dim: int
+    theta: float
+    frequencies: Optional[Tuple[float, ...]] = None
+
+    def __post_init__(self):
+        if self.rotary_dim % 2 or not 0 < self.rotary_dim <= self.head_dim:
+            raise ValueError(f"a rotation of {self.rotary_dim} of a head's {self.head_dim} channels: an even number within the head is needed")
+        if self.frequencies is not None and len(self.frequencies) != self.rotary_dim // 2:
+            raise ValueError(f"a rotation of {self.rotary_dim} channels needs {self.rotary_dim // 2} frequencies, not {len(self.frequencies)}")
+
+
+@dataclass(frozen=True)
 class RmsNormSpec:
     kind: ClassVar[str] = "rmsnorm"
     size: int
@@ -52,17 +69,56 @@ class AttentionSpec:
     o_proj: str
     position: Optional[Any] = None   # a position-encoding spec, or None for no rotation
     window: Optional[int] = None     # keys further back than this many positions are not seen
+    # What follows is absent (None) in the plain attention of a Llama layer; a layer that names any of it takes the general kernels.
+    value_dim: Optional[int] = None  # channels of a value head, where they differ from those of a query/key head
+    scale: Optional[float] = None    # what the scores are multiplied by; head_dim^(-1/2) if not given
+    chunk: Optional[int] = None      # position i sees j <= i only if floor(i / chunk) = floor(j / chunk), counted from the sequence's start
+    sinks: Optional[str] = None      # tensor [heads]: a learned score per head that joins the softmax's denominator and has no value
+    q_norm: Optional[str] = None     # tensors [head_dim]: RMS norm of every query (key) head with these weights, before the rotation
+    k_norm: Optional[str] = None
+    qk_norm_eps: float = 1e-6
+    head_gate: Optional[str] = None  # tensor [heads, hidden]: head h's output is multiplied by sigmoid(row h of it . the mixer's input)
+    keep_chunk: Optional[int] = None # the pages of chunks gone by are given back: set where this entry and every reader of its pages cut their masks alike
 
 
 @dataclass(frozen=True)
 class SwiGluSpec:
-    """down( silu(gate(x)) * up(x) ), no biases."""
+    """down( act(gate(x)) * up(x) ), no biases; act is SiLU, or the tanh form of GELU (`activation` = "gelu_tanh")."""
     kind: ClassVar[str] = "swiglu"
     hidden_size: int
     intermediate_size: int
     gate_proj: str
     up_proj: str
     down_proj: str
+    activation: str = "silu"
+
+
+@dataclass(frozen=True)
+class MlstmSpec:
+    """A matrix memory per head (the mLSTM of xLSTM) with exponential gating kept stable by a running maximum:
+        m_t = max(f_t + m_(t-1), i_t)
+        S_t = exp(f_t + m_(t-1) - m_t) S_(t-1) + exp(i_t - m_t) k_t v_t^T,   n_t the same with k_t alone
+        o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6)
+    with q scaled by key_dim^(-1/2), i = cap * tanh(pre_i / cap), f = logsigmoid(cap * tanh(pre_f / cap)), S, n, m zero at a
+    sequence's start.  Every head's o is divided by its root mean square; the heads side by side are multiplied by `out_norm`
+    and by sigmoid(gate(x)) and go through `o_proj`."""
+    kind: ClassVar[str] = "mlstm"
+    hidden_size: int
+    n_heads: int
+    key_dim: int
+    value_dim: int
+    gate_cap: float
+    norm_eps: float
+    q_proj: str
+    k_proj: str
+    v_proj: str
+    gate_proj: str
+    o_proj: str
+    out_norm: str
+    i_proj: str
+    i_bias: str
+    f_proj: str
+    f_bias: str
 
 
 @dataclass(frozen=True)
@@ -83,10 +139,12 @@ class SoftCapSpec:
 class LayerSpec:
     """One layer: which parts, and in which arrangement (`block`) they are wired."""
     mixer: Any
-    feed_forward: Any
+    feed_forward: Any                # None: the layer has no feed-forward half (blocks that allow it)
     mixer_norm: Any
     feed_forward_norm: Any
     block: str = "prenorm"
+    mixer_post_norm: Any = None      # "sandwich" blocks: a norm on what each half puts out, before it joins the residual stream
+    feed_forward_post_norm: Any = None
 
 
 @dataclass(frozen=True)

@@ -377,3 +377,137 @@ GI_API int gi_random_normal(void* out, int dtype, long n, unsigned long long key
     GI_CHECK_LAUNCH("random_normal");
     return 0;
 }
+
+// --------------------------------------------------------- a norm on a sublayer's output, added on
+// x[t, :] += w * (y[t, :] * rsqrt(mean(y[t, :]^2) + eps)): what a "sandwich" layer does with what its mixer or its
+// feed-forward puts out.  One workgroup per row; the sum of squares in 32-bit in an order that the row's length fixes.
+template <typename TW>
+__global__ __launch_bounds__(256) void rmsnorm_add_kernel(const float* __restrict__ y, const TW* __restrict__ w, float* __restrict__ x, int dim,
+                                                         float eps, size_t y_stride, size_t x_stride) {
+    __shared__ float red[4];
+    const float* yr = y + (size_t)blockIdx.x * y_stride;
+    float* xr = x + (size_t)blockIdx.x * x_stride;
+    float ss = 0.f;
+    for (int d = threadIdx.x; d < dim; d += 256) ss = fmaf(yr[d], yr[d], ss);
+    ss = block_sum<256>(ss, red);
+    const float scale = 1.0f / sqrtf(ss / (float)dim + eps);
+    for (int d = threadIdx.x; d < dim; d += 256) xr[d] += load_f32(w, d) * (scale * yr[d]);
+}
+
+GI_API int gi_rmsnorm_add(const float* y, const void* w, int w_dtype, float* x, int n_rows, int dim, float eps, long y_stride, long x_stride,
+                          hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && dim > 0 && y_stride >= dim && x_stride >= dim, "rmsnorm_add: bad sizes (rows %d, dim %d)", n_rows, dim);
+    if (w_dtype == GI_F32) rmsnorm_add_kernel<float><<<n_rows, 256, 0, stream>>>(y, (const float*)w, x, dim, eps, (size_t)y_stride, (size_t)x_stride);
+    else if (w_dtype == GI_BF16) rmsnorm_add_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(y, (const bf16_t*)w, x, dim, eps, (size_t)y_stride, (size_t)x_stride);
+    else return gi_fail("rmsnorm_add: unknown dtype %d", w_dtype);
+    GI_CHECK_LAUNCH("rmsnorm_add");
+    return 0;
+}
+
+// ------------------------------------------- head norm, rotation of a head's first channels, cache write
+// The general form of rope_store, one wave per (row, head):
+//   a query or key head is first divided by its root mean square and multiplied by `q_norm` / `k_norm` [hd] (if given),
+//   then the pairs (i, i + rot/2), i < rot/2, of its first `rot` channels are turned by the row's angles
+//   (cos, sin: [n_rows, rot/2]; nullptr or rot = 0: no rotation); the other channels pass;
+//   queries go to q_out [n_rows, n_heads*hd]; keys to the page's [kv_head][place][hd]; values, of `vd` channels a head,
+//   to the page's [kv_head][vd][place] behind all keys.  k == nullptr: another layer's pages are read and none written.
+constexpr int NRS_MAX_HD = 512;
+
+template <typename TQ, typename TC, typename TW>
+__global__ __launch_bounds__(64) void norm_rope_store_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
+                                                            long ldq, long ldk, long ldv, const TW* __restrict__ q_norm, const TW* __restrict__ k_norm,
+                                                            float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot,
+                                                            const int* __restrict__ pos, const int* __restrict__ slot, const int* __restrict__ table,
+                                                            int table_stride, TQ* __restrict__ q_out, TC* __restrict__ cache, long page_stride,
+                                                            int page_size, int n_heads, int n_kv, int hd, int vd) {
+    __shared__ float s[NRS_MAX_HD];
+    const int t = blockIdx.x, item = blockIdx.y, lane = threadIdx.x;
+    const int p = pos[t];
+    if (item >= n_heads + n_kv) {                      // a value head: copied into its page, transposed
+        const int h = item - n_heads - n_kv;
+        const long page = table[(size_t)slot[t] * table_stride + p / page_size];
+        TC* vbase = cache + page * page_stride + (size_t)n_kv * page_size * hd + (size_t)h * vd * page_size + p % page_size;
+        for (int d = lane; d < vd; d += 64) store_f32(vbase, (size_t)d * page_size, v[(size_t)t * ldv + h * vd + d]);
+        return;
+    }
+    const bool is_q = item < n_heads;
+    const int h = is_q ? item : item - n_heads;
+    const float* src = is_q ? q + (size_t)t * ldq + h * hd : k + (size_t)t * ldk + h * hd;
+    const TW* w = is_q ? q_norm : k_norm;
+    float ss = 0.f;
+    for (int d = lane; d < hd; d += 64) {
+        const float x = src[d];
+        s[d] = x;
+        ss = fmaf(x, x, ss);
+    }
+    if (w != nullptr) {
+        const float r = 1.0f / sqrtf(wave_sum(ss) / (float)hd + eps);
+        for (int d = lane; d < hd; d += 64) s[d] = load_f32(w, d) * (r * s[d]);
+    }
+    __syncthreads();
+    const int half = rot / 2;
+    const bool turn = cos_t != nullptr && rot > 0;
+    TC* kdst = nullptr;
+    TQ* qdst = nullptr;
+    if (is_q) qdst = q_out + ((size_t)t * n_heads + h) * hd;
+    else {
+        const long page = table[(size_t)slot[t] * table_stride + p / page_size];
+        kdst = cache + page * page_stride + ((size_t)h * page_size + p % page_size) * hd;
+    }
+    for (int d = lane; d < hd; d += 64) {
+        float out = s[d];
+        if (turn && d < rot) {
+            const int i = d < half ? d : d - half;
+            const float c = cos_t[(size_t)t * half + i], sn = sin_t[(size_t)t * half + i];
+            out = d < half ? s[d] * c - s[d + half] * sn : s[d] * c + s[d - half] * sn;
+        }
+        if (is_q) store_f32(qdst, d, out); else store_f32(kdst, d, out);
+    }
+}
+
+GI_API int gi_norm_rope_store(const float* q, const float* k, const float* v, long ldq, long ldk, long ldv, const void* q_norm, const void* k_norm,
+                              int norm_dtype, float eps, const float* cos_t, const float* sin_t, int rot, const int* pos, const int* slot,
+                              const int* table, int table_stride, void* q_out, int q_dtype, void* cache, int cache_dtype, long page_stride,
+                              int page_size, int n_rows, int n_heads, int n_kv, int hd, int vd, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && n_heads > 0 && n_kv > 0 && hd > 0 && hd <= NRS_MAX_HD && vd > 0, "norm_rope_store: bad sizes (rows %d heads %d kv %d hd %d vd %d)",
+               n_rows, n_heads, n_kv, hd, vd);
+    GI_REQUIRE((cos_t == nullptr) == (sin_t == nullptr) && rot >= 0 && rot % 2 == 0 && rot <= hd, "norm_rope_store: cos and sin go together, and the rotated channels are an even number within the head");
+    GI_REQUIRE(k == nullptr || (v != nullptr && cache != nullptr && table != nullptr && page_size > 0 && page_stride >= (long)n_kv * page_size * (hd + vd)),
+               "norm_rope_store: a cache write needs v, a cache, a table and a page stride of at least n_kv*page_size*(hd+vd)");
+    GI_REQUIRE(n_heads + 2 * n_kv <= 65535, "norm_rope_store: too many heads");
+    dim3 grid(n_rows, n_heads + (k ? 2 * n_kv : 0));
+#define LAUNCH(TQ, TC, TW)                                                                                                                    \
+    norm_rope_store_kernel<TQ, TC, TW><<<grid, 64, 0, stream>>>(q, k, v, ldq, ldk, ldv, (const TW*)q_norm, (const TW*)k_norm, eps, cos_t, sin_t, rot, pos, \
+                                                                slot, table, table_stride, (TQ*)q_out, (TC*)cache, page_stride, page_size, n_heads, n_kv, hd, vd)
+    if (q_dtype == GI_F32 && cache_dtype == GI_F32 && norm_dtype == GI_F32) LAUNCH(float, float, float);
+    else if (q_dtype == GI_BF16 && cache_dtype == GI_BF16 && norm_dtype == GI_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);
+    else if (q_dtype == GI_BF16 && cache_dtype == GI_BF16 && norm_dtype == GI_F32) LAUNCH(bf16_t, bf16_t, float);
+    else return gi_fail("norm_rope_store: dtypes (%d, %d, %d) are not served", q_dtype, cache_dtype, norm_dtype);
+#undef LAUNCH
+    GI_CHECK_LAUNCH("norm_rope_store");
+    return 0;
+}
+
+// -------------------------------------------------------------------- gated feed-forward, by activation
+// h[t, i] = act(gu[t, i]) * gu[t, inter + i]; act 0: SiLU, 1: the tanh form of GELU,
+// 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).
+template <typename TO>
+__global__ void act_mul_kernel(const float* __restrict__ gu, TO* __restrict__ h, int inter, size_t n, int act) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const size_t t = i / inter, c = i % inter;
+    const float g = gu[t * 2 * inter + c], u = gu[t * 2 * inter + inter + c];
+    const float a = act == 0 ? g * (1.0f / (1.0f + expf(-g))) : 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+    store_f32(h, i, a * u);
+}
+
+GI_API int gi_act_mul(const float* gate_up, void* h, int h_dtype, int n_rows, int inter, int act, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && inter > 0 && (act == 0 || act == 1), "act_mul: n_rows %d and inter %d must be positive, the activation 0 or 1", n_rows, inter);
+    const size_t n = (size_t)n_rows * inter;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (h_dtype == GI_F32) act_mul_kernel<float><<<blocks, 256, 0, stream>>>(gate_up, (float*)h, inter, n, act);
+    else if (h_dtype == GI_BF16) act_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>(gate_up, (bf16_t*)h, inter, n, act);
+    else return gi_fail("act_mul: unknown dtype %d", h_dtype);
+    GI_CHECK_LAUNCH("act_mul");
+    return 0;
+}

@@ -43,7 +43,7 @@ class _CacheView:
             from ..cache import PagedKvNeed, StateNeed
             if isinstance(need, PagedKvNeed):
                 kv, table, _ = manager.kv(i)
-                self._layer.append(LayerCache(kv=kv, table=table, writes=src is None))
+                self._layer.append(LayerCache(kv=kv, table=table, writes=src is None, page_size=manager.page_size))
             elif isinstance(need, StateNeed):
                 self._layer.append(LayerCache(state=manager.state(i)))
             else:

@@ -35,7 +35,15 @@ _SIGNATURES = {
     "gi_softcap_rows": [c_void_p, c_int, c_int, c_long, c_float, c_void_p],
     "gi_gemm_exact": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p],
     "gi_attention_exact": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int,
-                           c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+                           c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_long, c_void_p],
+    "gi_rmsnorm_add": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_long, c_long, c_void_p],
+    "gi_norm_rope_store": [c_void_p, c_void_p, c_void_p, c_long, c_long, c_long, c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int,
+                           c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "gi_act_mul": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "gi_segments": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p],
+    "gi_mlstm_scan": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_int, c_void_p,
+                      c_void_p, c_long, c_void_p, c_long, c_int, c_int, c_int, c_void_p],
+    "gi_head_norm_gate": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_float, c_void_p],
     "gi_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long, c_void_p],
     "gi_attention_prompt_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
                                  c_float, c_int, c_void_p, c_void_p, c_int, c_void_p, c_long, c_void_p],
@@ -87,6 +95,10 @@ def lib():
         l.gi_compute_units.restype = c_int
         l.gi_gemm_bf16_qkv_rope_store_max_parts.argtypes = [c_int, c_int, c_int]
         l.gi_gemm_bf16_qkv_rope_store_max_parts.restype = c_int
+        l.gi_mlstm_state_floats.argtypes = [c_int, c_int, c_int]
+        l.gi_mlstm_state_floats.restype = c_long
+        l.gi_mlstm_max_key_dim.argtypes = []
+        l.gi_mlstm_max_key_dim.restype = c_int
         l.gi_probe_mfma_flops.argtypes = [c_int, c_int]
         l.gi_probe_mfma_flops.restype = c_long
         _lib = l
@@ -398,19 +410,171 @@ def attention_max_head_size() -> int:
     return lib().gi_attention_exact_max_head_size()
 
 
-def attention_exact(q, cache, out, positions, slots, table, n_heads, n_kv, hd, window=None, scale=None):
-    """Each row attends over its request's cached keys up to its own position."""
-    _dev(q, cache, out, positions, slots, table)
+def _check_paged(cache, table, what):
+    """A layer's pages as the general kernels take them: [pages, ...] with whole pages contiguous, whatever the axes behind."""
+    if not (cache.dim() >= 2 and cache[0].is_contiguous()):
+        raise KernelError(f"{what}: the pages must each be contiguous")
+    if not (table.dim() == 2 and table.dtype == torch.int32 and table.stride(1) == 1):
+        raise KernelError(f"{what}: the page table must be int32 [slots, pages]")
+
+
+def attention_exact(q, cache, out, positions, slots, table, n_heads, n_kv, hd, window=None, scale=None, *, page_size=None, value_dim=None,
+                    chunk=None, sinks=None, gate=None):
+    """Each row attends over its request's cached keys up to its own position, no further back than `window` positions and not
+    beyond the start of its own chunk of `chunk` positions.  value_dim: channels of a value head (hd if not given); sinks:
+    float32 [heads], a score per head that joins the softmax's denominator only; gate: float32 [n, >= heads] (unit inner
+    stride), head h's output is multiplied by sigmoid(gate[t, h])."""
+    _dev(q, cache, out, positions, slots, table, sinks, gate)
     n = q.shape[0]
-    if not (q.shape == (n, n_heads * hd) and q.is_contiguous() and out.shape == q.shape and out.is_contiguous()):
-        raise KernelError( "attention: q and out must be [n, heads*hd], contiguous")
-    page_size = cache.shape[3]
-    _check_cache(cache, table, page_size, n_kv, hd, "attention")
+    vd = int(value_dim or hd)
+    if not (q.shape == (n, n_heads * hd) and q.is_contiguous() and out.shape == (n, n_heads * vd) and out.is_contiguous()):
+        raise KernelError("attention: q must be [n, heads*hd] and out [n, heads*vd], contiguous")
+    if page_size is None:
+        page_size = cache.shape[3]
+        _check_cache(cache, table, page_size, n_kv, hd, "attention")
+    else:
+        _check_paged(cache, table, "attention")
+    if sinks is not None and not (sinks.dtype == torch.float32 and sinks.is_contiguous() and sinks.numel() == n_heads):
+        raise KernelError("attention: sinks must be float32 [heads]")
+    if gate is not None and not (gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape[0] == n and gate.shape[1] >= n_heads and gate.stride(1) == 1):
+        raise KernelError("attention: the heads' gates must be float32 [n, heads] with unit inner stride")
     _i32(positions, "attention: positions", n)
     _i32(slots, "attention: slots", n)
     _call("gi_attention_exact", q.data_ptr(), _code(q, "attention: q"), cache.data_ptr(), _code(cache, "attention: cache"), out.data_ptr(),
           _code(out, "attention: out"), positions.data_ptr(), slots.data_ptr(), table.data_ptr(), table.stride(0), cache.stride(0),
-          page_size, n, n_heads, n_kv, hd, int(window or 0), float(scale if scale is not None else hd ** -0.5), _stream())
+          page_size, n, n_heads, n_kv, hd, vd, int(window or 0), int(chunk or 0), float(scale if scale is not None else hd ** -0.5),
+          _ptr(sinks), _ptr(gate), gate.stride(0) if gate is not None else 0, _stream())
+    return out
+
+
+def rmsnorm_add(y, weight, eps, x):
+    """x += weight * (y * rsqrt(mean(y^2) + eps)) per row; x and y float32 [n, dim]."""
+    _dev(y, weight, x)
+    n, dim = x.shape
+    if not (x.dtype == torch.float32 and y.dtype == torch.float32 and y.shape == (n, dim) and x.stride(1) == 1 and y.stride(1) == 1):
+        raise KernelError("rmsnorm_add: x and y must be float32 [n, dim] with unit inner stride")
+    if not (weight.shape == (dim,) and weight.is_contiguous()):
+        raise KernelError("rmsnorm_add: weight must be [dim]")
+    _call("gi_rmsnorm_add", y.data_ptr(), weight.data_ptr(), _code(weight, "rmsnorm_add: weight"), x.data_ptr(), n, dim, float(eps), y.stride(0), x.stride(0), _stream())
+    return x
+
+
+def norm_rope_store(q, k, v, q_norm, k_norm, eps, cos, sin, rotary_dim, positions, slots, table, q_out, cache, page_size, n_heads, n_kv, hd, vd):
+    """The general form of `rope_store`: every query and key head is first RMS-normed with q_norm / k_norm [hd] (None: not), then
+    the pairs (i, i + rotary_dim/2) of its first rotary_dim channels are turned (cos, sin float32 [n, rotary_dim/2]; None: not);
+    queries go to q_out, keys and the values (vd channels a head) into the cache's pages.  k None: the pages are another layer's."""
+    _dev(q, k, v, q_norm, k_norm, cos, sin, positions, slots, table, q_out, cache)
+    n = q.shape[0]
+    if not (q.dtype == torch.float32 and q.shape[1] == n_heads * hd and q.stride(1) == 1 and q_out.shape == (n, n_heads * hd) and q_out.is_contiguous()):
+        raise KernelError("norm_rope_store: q must be float32 [n, heads*hd] and q_out [n, heads*hd], contiguous")
+    half = int(rotary_dim) // 2 if cos is not None else 0
+    if cos is not None:
+        for t in (cos, sin):
+            if not (t.dtype == torch.float32 and t.shape == (n, half) and t.is_contiguous()):
+                raise KernelError("norm_rope_store: cos/sin must be float32 [n, rotary_dim/2]")
+    norm_code = None
+    for w in (q_norm, k_norm):
+        if w is not None:
+            if not (w.shape == (hd,) and w.is_contiguous() and (norm_code is None or norm_code == _code(w, "norm_rope_store: norm"))):
+                raise KernelError("norm_rope_store: the heads' norm weights must be [hd], of one dtype")
+            norm_code = _code(w, "norm_rope_store: norm")
+    if k is not None:
+        if not (k.dtype == torch.float32 and k.shape == (n, n_kv * hd) and k.stride(1) == 1 and v.dtype == torch.float32 and v.shape == (n, n_kv * vd) and v.stride(1) == 1):
+            raise KernelError("norm_rope_store: k must be float32 [n, kv_heads*hd] and v [n, kv_heads*vd]")
+        _check_paged(cache, table, "norm_rope_store")
+        if cache.stride(0) < n_kv * page_size * (hd + vd):
+            raise KernelError("norm_rope_store: the pages are too small for these heads")
+    _i32(positions, "norm_rope_store: positions", n)
+    _i32(slots, "norm_rope_store: slots", n)
+    cache_code = _code(cache, "norm_rope_store: cache") if k is not None else _code(q_out, "norm_rope_store: q_out")
+    _call("gi_norm_rope_store", q.data_ptr(), _ptr(k), _ptr(v), q.stride(0), k.stride(0) if k is not None else 0, v.stride(0) if v is not None else 0,
+          _ptr(q_norm), _ptr(k_norm), norm_code if norm_code is not None else F32, float(eps), _ptr(cos), _ptr(sin), 2 * half, positions.data_ptr(),
+          slots.data_ptr(), _ptr(table) if k is not None else None, table.stride(0) if k is not None else 0, q_out.data_ptr(),
+          _code(q_out, "norm_rope_store: q_out"), _ptr(cache) if k is not None else None, cache_code, cache.stride(0) if k is not None else 0,
+          int(page_size), n, n_heads, n_kv, hd, vd, _stream())
+
+
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def act_mul(gate_up, out, activation="silu"):
+    """out[t, i] = act(gate_up[t, i]) * gate_up[t, inter + i]; act "silu" or "gelu_tanh" (the tanh form of GELU)."""
+    _dev(gate_up, out)
+    n, inter = out.shape
+    if activation not in ACTIVATIONS:
+        raise KernelError(f"act_mul: unknown activation {activation!r}; known: {', '.join(ACTIVATIONS)}")
+    if not (gate_up.dtype == torch.float32 and gate_up.shape == (n, 2 * inter) and gate_up.is_contiguous() and out.is_contiguous()):
+        raise KernelError("act_mul: gate_up must be float32 [n, 2*inter], out contiguous")
+    _call("gi_act_mul", gate_up.data_ptr(), out.data_ptr(), _code(out, "act_mul: out"), n, inter, ACTIVATIONS[activation], _stream())
+    return out
+
+
+def segments(ctx):
+    """(first row, number of rows) of every request of the step as int32 device tensors [requests], made on the device from the
+    rows' slots and positions (a run of rows ends where the slot changes or the position does not follow): nothing of it comes
+    from the host but the number of requests, so a captured pass may use it.  Made once per step, kept in ctx.memo."""
+    if "segments" not in ctx.memo:
+        n_segs = len(ctx.seg_len)
+        both = torch.empty((2, n_segs), dtype=torch.int32, device=ctx.device)
+        _i32(ctx.row_slot, "segments: slots", ctx.n_rows)
+        _i32(ctx.row_pos, "segments: positions", ctx.n_rows)
+        _call("gi_segments", ctx.row_slot.data_ptr(), ctx.row_pos.data_ptr(), ctx.n_rows, both[0].data_ptr(), both[1].data_ptr(), n_segs, _stream())
+        ctx.memo["segments"] = (both[0], both[1])
+    return ctx.memo["segments"]
+
+
+def mlstm_state_floats(n_heads, dk, dv) -> int:
+    """32-bit numbers of one request's matrix memories, as `mlstm_scan` lays them out for itself: per head and tile of 64 value
+    channels the tile of S, n padded to a multiple of 4, m and 3 unused (the library's `gi_mlstm_state_floats` says the same; this
+    one needs no library, so that a cache can be planned without one)."""
+    return n_heads * (-(-dv // 64)) * (dk * 64 + ((dk + 3) & ~3) + 4)
+
+
+MLSTM_MAX_KEY_DIM = 256
+
+
+def mlstm_max_key_dim() -> int:
+    return MLSTM_MAX_KEY_DIM
+
+
+def mlstm_scan(proj, offsets, i_bias, f_bias, cap, q_scale, seg_start, seg_len, row_slot, state, out, n_heads, dk, dv):
+    """The matrix memories of a step's requests stepped over the requests' rows, in order (csrc/recurrent.hip states the recurrence).
+    proj: float32 [n, columns]; offsets = the first columns of (q, k, v, i, f) in it; out: float32 [n, heads*dv];
+    state: float32 [slots, mlstm_state_floats], read at each request's first row of the step and written after its last."""
+    _dev(proj, i_bias, f_bias, seg_start, seg_len, row_slot, state, out)
+    n = proj.shape[0]
+    q_off, k_off, v_off, i_off, f_off = (int(o) for o in offsets)
+    if not (proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and out.dtype == torch.float32 and out.shape == (n, n_heads * dv) and out.stride(1) == 1):
+        raise KernelError("mlstm_scan: proj must be float32 [n, columns] and out float32 [n, heads*dv]")
+    if max(q_off + n_heads * dk, k_off + n_heads * dk, v_off + n_heads * dv, i_off + n_heads, f_off + n_heads) > proj.shape[1] or min(q_off, k_off, v_off, i_off, f_off) < 0:
+        raise KernelError("mlstm_scan: the columns named lie outside proj")
+    for t, name in ((i_bias, "i_bias"), (f_bias, "f_bias")):
+        if not (t.dtype == torch.float32 and t.is_contiguous() and t.numel() == n_heads):
+            raise KernelError(f"mlstm_scan: {name} must be float32 [heads]")
+    n_segs = seg_start.numel()
+    _i32(seg_start, "mlstm_scan: seg_start", n_segs)
+    _i32(seg_len, "mlstm_scan: seg_len", n_segs)
+    _i32(row_slot, "mlstm_scan: slots", n)
+    if not (state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1 and state.shape[1] >= mlstm_state_floats(n_heads, dk, dv)):
+        raise KernelError("mlstm_scan: state must be float32 [slots, mlstm_state_floats]")
+    _call("gi_mlstm_scan", proj.data_ptr(), proj.stride(0), q_off, k_off, v_off, i_off, f_off, i_bias.data_ptr(), f_bias.data_ptr(), float(cap), float(q_scale),
+          seg_start.data_ptr(), seg_len.data_ptr(), n_segs, row_slot.data_ptr(), state.data_ptr(), state.stride(0), out.data_ptr(), out.stride(0),
+          n_heads, dk, dv, _stream())
+    return out
+
+
+def head_norm_gate(o, gate, weight, eps, out, n_heads, dv):
+    """out[t, h*dv + d] = weight[h*dv + d] * o[t, h, d] * rsqrt(mean over d of o[t, h, :]^2 + eps) * sigmoid(gate[t, h*dv + d]);
+    o and gate float32 [n, heads*dv] (unit inner stride: columns of a wider product are fine)."""
+    _dev(o, gate, weight, out)
+    n = o.shape[0]
+    for t, name in ((o, "o"), (gate, "gate")):
+        if not (t.dtype == torch.float32 and t.shape == (n, n_heads * dv) and t.stride(1) == 1):
+            raise KernelError(f"head_norm_gate: {name} must be float32 [n, heads*dv]")
+    if not (weight.numel() == n_heads * dv and weight.is_contiguous() and out.shape == (n, n_heads * dv) and out.stride(1) == 1):
+        raise KernelError("head_norm_gate: weight must be [heads*dv] and out [n, heads*dv]")
+    _call("gi_head_norm_gate", o.data_ptr(), o.stride(0), gate.data_ptr(), gate.stride(0), weight.data_ptr(), _code(weight, "head_norm_gate: weight"),
+          out.data_ptr(), _code(out, "head_norm_gate: out"), out.stride(0), n, n_heads, dv, float(eps), _stream())
     return out
 
 
@@ -679,6 +843,13 @@ def attention(q, cache, out, ctx, table, n_heads, n_kv, hd, window=None):
         if (not plan.n_tiles or attention_bf16_supports(hd, page_size, True)) and (not plan.n_decode or attention_bf16_supports(hd, page_size, False)):
             return attention_bf16(q, cache, out, plan, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window)
     return attention_exact(q, cache, out, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window)
+
+
+def attention_general(q, cache, out, ctx, table, n_heads, n_kv, hd, *, page_size, value_dim=None, window=None, chunk=None, scale=None, sinks=None, gate=None):
+    """Attention of a step's rows for layers with any of: value heads of another size, a scale of their own, a mask cut into
+    chunks, sinks, a gate per head."""
+    return attention_exact(q, cache, out, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window, scale, page_size=page_size,
+                           value_dim=value_dim, chunk=chunk, sinks=sinks, gate=gate)
 
 
 # Up to so many rows the decode kernel rotates and writes the pages itself.  It saves the rotation kernel's launch wherever the

@@ -76,9 +76,21 @@ def qkv_rotate_store_attend(h, w_qkv, ctx, cache, *, n_heads, n_kv_heads, head_d
     return att
 
 
+def _pad_rows(w, multiple=16):
+    """The stacked matrix with rows of zeros behind it up to a multiple of `multiple` (so that the product's 32-bit rows start at
+    multiples of 16 bytes)."""
+    extra = -w.shape[0] % multiple
+    return w if not extra else torch.cat([w, torch.zeros((extra, w.shape[1]), dtype=w.dtype, device=w.device)], dim=0).contiguous()
+
+
 class Attention(Mixer):
+    """Plain (Llama) attention takes the kernels chosen in `qkv_rotate_store_attend`.  A spec that names any of the further
+    features (value heads of another size, a scale of its own, a mask cut into chunks, sinks, norms on query and key heads, a
+    gate per head, a rotation of a part of the head) takes the general path: one product with [q; k; v; head gates], one kernel
+    that norms, turns and stores, and the attention kernel that knows all of these."""
     accepts_deferred_norm = True      # its input goes into `linear` only
     hands_norm_on = True              # `forward` takes `then`, the norm that reads the residual next
+    can_overwrite = True              # `forward(..., overwrite=True)` stores its result in `residual` instead of adding onto it
 
     def __init__(self, spec, tensors, dtype, device):
         super().__init__(spec, tensors, dtype, device)
@@ -88,25 +100,57 @@ class Attention(Mixer):
         if not 0 < s.head_dim <= ops.attention_max_head_size():
             raise ValueError(f"attention: head_dim = {s.head_dim} is outside what the attention kernels take (1 to {ops.attention_max_head_size()} channels a head)")
         self.a_dim, self.kv_dim = s.n_heads * s.head_dim, s.n_kv_heads * s.head_dim
-        self.w_qkv = torch.cat([tensors[s.q_proj], tensors[s.k_proj], tensors[s.v_proj]], dim=0).contiguous()
-        self.w_o = tensors[s.o_proj]
+        self.value_dim = s.value_dim or s.head_dim
+        self.general = self._is_general(s)
         self.position = None if s.position is None else position_class(s.position)(s.position, tensors, dtype, device)
+        if not 0 < self.value_dim <= ops.attention_max_head_size():
+            raise ValueError(f"attention: value heads of {self.value_dim} channels are outside what the attention kernels take")
+        if self.general:
+            stacked = [tensors[s.q_proj]] + ([tensors[s.k_proj], tensors[s.v_proj]] if s.k_proj is not None else [])
+            self.gate_at = sum(w.shape[0] for w in stacked)
+            if s.head_gate is not None:
+                stacked.append(tensors[s.head_gate])
+            self.w_qkv = _pad_rows(torch.cat(stacked, dim=0).contiguous())
+            self.sinks = None if s.sinks is None else tensors[s.sinks].float().contiguous()
+            self.q_norm = None if s.q_norm is None else tensors[s.q_norm]
+            self.k_norm = None if s.k_norm is None else tensors[s.k_norm]
+            if self.position is not None and not (hasattr(self.position, "partial_tables") or type(self.position).half_split_tables is not PositionEncoding.half_split_tables):
+                if self.q_norm is not None or self.k_norm is not None:
+                    raise ValueError("attention: norms on query and key heads come before the rotation, which needs a position encoding that hands over its cosines and sines")
+        else:
+            self.w_qkv = torch.cat([tensors[s.q_proj], tensors[s.k_proj], tensors[s.v_proj]], dim=0).contiguous()
+        self.w_o = tensors[s.o_proj]
         self.in_dtype = activation_dtype_for(self.w_qkv, dtype)
         self.att_dtype = activation_dtype_for(self.w_o, dtype)
         self.graph_safe = self.position is None or bool(getattr(self.position, "graph_safe", False))
 
+    @staticmethod
+    def _is_general(s) -> bool:
+        return (s.k_proj is None or any(v is not None for v in (s.value_dim, s.scale, s.chunk, s.sinks, s.q_norm, s.k_norm, s.head_gate))
+                or getattr(s.position, "kind", None) == "rotary_partial")
+
     @classmethod
     def tensor_needs(cls, spec):
-        a, kv, d = spec.n_heads * spec.head_dim, spec.n_kv_heads * spec.head_dim, spec.hidden_size
-        return [TensorNeed(spec.q_proj, (a, d)), TensorNeed(spec.k_proj, (kv, d)), TensorNeed(spec.v_proj, (kv, d)),
-                TensorNeed(spec.o_proj, (d, a))]
+        a, kv, d, vd = spec.n_heads * spec.head_dim, spec.n_kv_heads * spec.head_dim, spec.hidden_size, spec.value_dim or spec.head_dim
+        needs = [TensorNeed(spec.q_proj, (a, d)), TensorNeed(spec.o_proj, (d, spec.n_heads * vd))]
+        if spec.k_proj is not None:            # (a layer that reads another layer's pages has no keys and values of its own)
+            needs += [TensorNeed(spec.k_proj, (kv, d)), TensorNeed(spec.v_proj, (spec.n_kv_heads * vd, d))]
+        if spec.q_norm is not None:
+            needs.append(TensorNeed(spec.q_norm, (spec.head_dim,), "norm"))
+        if spec.k_norm is not None and spec.k_proj is not None:
+            needs.append(TensorNeed(spec.k_norm, (spec.head_dim,), "norm"))
+        if spec.sinks is not None:
+            needs.append(TensorNeed(spec.sinks, (spec.n_heads,)))
+        if spec.head_gate is not None:
+            needs.append(TensorNeed(spec.head_gate, (spec.n_heads, d)))
+        return needs
 
     @classmethod
     def cache_need(cls, spec):
-        return PagedKvNeed(spec.n_kv_heads, spec.head_dim, spec.window)
+        return PagedKvNeed(spec.n_kv_heads, spec.head_dim, spec.window, None if spec.value_dim in (None, spec.head_dim) else spec.value_dim, spec.keep_chunk)
 
     def takes_handed_norm(self, n_rows: int) -> bool:
-        if self.in_dtype != torch.bfloat16:
+        if self.in_dtype != torch.bfloat16 or self.general:
             return False
         if ops.gemm_bf16_takes_norm(n_rows, self.w_qkv.shape[0], self.w_qkv.shape[1]):
             return True
@@ -114,8 +158,39 @@ class Attention(Mixer):
         half_split = self.position is None or getattr(type(self.position), "half_split_tables", None) is not PositionEncoding.half_split_tables
         return half_split and ops.gemm_bf16_qkv_rope_store_takes(n_rows, self.w_qkv.shape[0], self.w_qkv.shape[1], self.spec.head_dim)
 
-    def forward(self, h, residual, ctx, cache, then=None):
+    def _attend_general(self, h, ctx, cache):
+        """The heads' outputs [rows, heads * value_dim] by the general path."""
+        from .rope import rotation_tables
+        s, T, vd = self.spec, ctx.n_rows, self.value_dim
+        proj = torch.empty((T, self.w_qkv.shape[0]), dtype=torch.float32, device=ctx.device)
+        linear(h, self.w_qkv, proj)
+        q, k, v = proj[:, :self.a_dim], None, None
+        if s.k_proj is not None and cache.writes:
+            k, v = proj[:, self.a_dim:self.a_dim + self.kv_dim], proj[:, self.a_dim + self.kv_dim:self.a_dim + self.kv_dim + s.n_kv_heads * vd]
+        gate = proj[:, self.gate_at:self.gate_at + s.n_heads] if s.head_gate is not None else None
+        tables = rotation_tables(self.position, ctx)
+        if self.position is not None and tables is None:          # an encoding with kernels of its own turns q and k in place
+            self.position.apply(q, k, ctx, s.n_heads, s.n_kv_heads, s.head_dim)
+        cos, sin, turned = tables if tables is not None else (None, None, 0)
+        q_ready = torch.empty((T, self.a_dim), dtype=cache.kv.dtype, device=ctx.device)
+        ops.norm_rope_store(q, k, v, self.q_norm, self.k_norm if k is not None else None, s.qk_norm_eps, cos, sin, turned, ctx.row_pos, ctx.row_slot,
+                            cache.table, q_ready, cache.kv, cache.page_size, s.n_heads, s.n_kv_heads, s.head_dim, vd)
+        att = torch.empty((T, s.n_heads * vd), dtype=cache.kv.dtype, device=ctx.device)
+        return ops.attention_general(q_ready, cache.kv, att, ctx, cache.table, s.n_heads, s.n_kv_heads, s.head_dim, page_size=cache.page_size,
+                                     value_dim=vd, window=s.window, chunk=s.chunk, scale=s.scale, sinks=self.sinks, gate=gate)
+
+    def forward(self, h, residual, ctx, cache, then=None, overwrite=False):
         s = self.spec
+        if self.general:
+            att = self._attend_general(h, ctx, cache)
+            if att.dtype != self.att_dtype:
+                att = att.to(self.att_dtype)
+            if overwrite:
+                linear(att, self.w_o, residual)
+                return None
+            return linear_onto(att, self.w_o, residual, then)
+        if overwrite:
+            residual.zero_()
         att = qkv_rotate_store_attend(h, self.w_qkv, ctx, cache, n_heads=s.n_heads, n_kv_heads=s.n_kv_heads, head_dim=s.head_dim,
                                       position=self.position, window=s.window, in_dtype=self.in_dtype)
         if att.dtype != self.att_dtype:

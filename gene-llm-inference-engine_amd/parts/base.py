@@ -71,7 +71,8 @@ class StepContext:
 @dataclass
 class LayerCache:
     """A run-order entry's view of the cache manager."""
-    kv: Optional[torch.Tensor] = None        # [page, 2, kv_head, place, head_dim] of this layer
+    kv: Optional[torch.Tensor] = None        # [page, 2, kv_head, place, head_dim] of this layer ([page, numbers] where value heads have another size than key heads)
+    page_size: int = 0                       # positions a page holds
     table: Optional[torch.Tensor] = None     # int32 [slot, pages]
     state: Optional[torch.Tensor] = None     # [slot, ...] fixed-size state
     writes: bool = True                      # False: the pages belong to another entry, read only

@@ -2,9 +2,14 @@
 
 "prenorm" (reference: src/model/transformer.cpp:385-450):
     x += mixer(norm_1(x));  x += feed_forward(norm_2(x))
+"sandwich": a norm before and a norm after each half; the feed-forward half may be absent:
+    x += post_1(mixer(norm_1(x)));  x += post_2(feed_forward(norm_2(x)))
 The residual stream x is float32 [T, hidden] and is changed in place."""
 from __future__ import annotations
 
+import torch
+
+from ..kernels import ops
 from .base import feed_forward_class, mixer_class, norm_class, register_block
 from .norm import norm_to_hand_on
 
@@ -71,3 +76,69 @@ class PreNormBlock:
 
 
 register_block("prenorm", PreNormBlock)
+
+
+class SandwichBlock:
+    """x += post_1(mixer(norm_1(x))), then, if the layer has a feed-forward, x += post_2(feed_forward(norm_2(x))).  A half's
+    result goes into rows of its own (a part that `can_overwrite` stores it there, any other part adds onto zeros), and the
+    norm behind the half adds the normed rows onto x in one kernel where it is an RMS norm with weights."""
+
+    def __init__(self, spec, tensors, dtype, device):
+        self.spec = spec
+        build = lambda s: None if s is None else norm_class(s)(s, tensors, dtype, device)
+        if spec.mixer_post_norm is None or (spec.feed_forward is not None and (spec.feed_forward_norm is None or spec.feed_forward_post_norm is None)):
+            raise ValueError("a sandwich layer needs a norm before and behind each of its halves")
+        self.mixer_norm, self.mixer_post_norm = build(spec.mixer_norm), build(spec.mixer_post_norm)
+        self.mixer = mixer_class(spec.mixer)(spec.mixer, tensors, dtype, device)
+        self.feed_forward = None
+        if spec.feed_forward is not None:
+            self.feed_forward_norm, self.feed_forward_post_norm = build(spec.feed_forward_norm), build(spec.feed_forward_post_norm)
+            self.feed_forward = feed_forward_class(spec.feed_forward)(spec.feed_forward, tensors, dtype, device)
+
+    def _parts(self):
+        halves = [self.mixer_norm, self.mixer, self.mixer_post_norm]
+        return halves + ([self.feed_forward_norm, self.feed_forward, self.feed_forward_post_norm] if self.feed_forward is not None else [])
+
+    @property
+    def graph_safe(self):
+        return all(getattr(p, "graph_safe", False) for p in self._parts())
+
+    @classmethod
+    def tensor_needs(cls, spec):
+        needs = []
+        for s in (spec.mixer_norm, spec.mixer_post_norm) + ((spec.feed_forward_norm, spec.feed_forward_post_norm) if spec.feed_forward is not None else ()):
+            needs += norm_class(s).tensor_needs(s)
+        needs += mixer_class(spec.mixer).tensor_needs(spec.mixer)
+        if spec.feed_forward is not None:
+            needs += feed_forward_class(spec.feed_forward).tensor_needs(spec.feed_forward)
+        return needs
+
+    @classmethod
+    def cache_need(cls, spec):
+        return mixer_class(spec.mixer).cache_need(spec.mixer)
+
+    @staticmethod
+    def _half(norm, part, post, x, ctx, *cache):
+        h = PreNormBlock._normed(norm, part, x, ctx)
+        if getattr(part, "can_overwrite", False):
+            y = torch.empty_like(x)
+            part.forward(h, y, ctx, *cache, overwrite=True)
+        else:
+            y = torch.zeros_like(x)
+            part.forward(h, y, ctx, *cache)
+        if hasattr(post, "add_onto"):
+            post.add_onto(y, x)
+        else:
+            x += post(y, torch.float32)
+
+    def forward(self, x, ctx, cache):
+        self._half(self.mixer_norm, self.mixer, self.mixer_post_norm, x, ctx, cache)
+        if ctx.trace is not None:
+            ctx.trace("attn_out", x)
+        if self.feed_forward is not None:
+            self._half(self.feed_forward_norm, self.feed_forward, self.feed_forward_post_norm, x, ctx)
+        if ctx.trace is not None:
+            ctx.trace("ffn_out", x)
+
+
+register_block("sandwich", SandwichBlock)

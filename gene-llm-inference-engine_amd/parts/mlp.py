@@ -1,6 +1,6 @@
-"""SwiGLU feed-forward: residual += down( silu(gate(h)) * up(h) ), silu(g) = g / (1 + exp(-g))
-(reference: src/model/transformer.cpp:437-450).  gate and up run as one product with the stacked
-matrix [gate; up]."""
+"""Gated feed-forward: residual += down( act(gate(h)) * up(h) ); act is SiLU, silu(g) = g / (1 + exp(-g))
+(SwiGLU; reference: src/model/transformer.cpp:437-450), or the tanh form of GELU where the spec says so.  gate and up run
+as one product with the stacked matrix [gate; up]; with SiLU and bfloat16 the gate is applied inside that product."""
 from __future__ import annotations
 
 import torch
@@ -15,6 +15,7 @@ class SwiGlu(FeedForward):
     graph_safe = True
     accepts_deferred_norm = True      # its input goes into `linear` only
     hands_norm_on = True              # `forward` takes `then`, the norm that reads the residual next
+    can_overwrite = True              # `forward(..., overwrite=True)` stores its result in `residual` instead of adding onto it
 
     def __init__(self, spec, tensors, dtype, device):
         super().__init__(spec, tensors, dtype, device)
@@ -23,7 +24,10 @@ class SwiGlu(FeedForward):
         self.in_dtype = activation_dtype_for(gate, dtype)
         self.mid_dtype = activation_dtype_for(self.w_down, dtype)
         # bfloat16 throughout: the gate is applied inside the product (weights interleaved for it)
-        self.fused = (self.in_dtype == torch.bfloat16 and self.mid_dtype == torch.bfloat16 and up.dtype == torch.bfloat16
+        self.activation = getattr(spec, "activation", "silu")
+        if self.activation not in ops.ACTIVATIONS:
+            raise ValueError(f"feed-forward: unknown activation {self.activation!r}; known: {', '.join(ops.ACTIVATIONS)}")
+        self.fused = (self.activation == "silu" and self.in_dtype == torch.bfloat16 and self.mid_dtype == torch.bfloat16 and up.dtype == torch.bfloat16
                       and spec.intermediate_size % 16 == 0 and spec.hidden_size % 8 == 0)
         self.w_gate_up = ops.interleave_gate_up(gate, up) if self.fused else torch.cat([gate, up], dim=0).contiguous()
 
@@ -35,16 +39,19 @@ class SwiGlu(FeedForward):
     def takes_handed_norm(self, n_rows: int) -> bool:
         return self.in_dtype == torch.bfloat16 and ops.gemm_bf16_takes_norm(n_rows, self.w_gate_up.shape[0], self.w_gate_up.shape[1], self.fused)
 
-    def forward(self, h, residual, ctx, then=None):
+    def forward(self, h, residual, ctx, then=None, overwrite=False):
         T, inter = ctx.n_rows, self.spec.intermediate_size
         if self.fused:
             mid = torch.empty((T, inter), dtype=torch.bfloat16, device=ctx.device)
             linear(h, self.w_gate_up, mid, gated=True)
-            return linear_onto(mid, self.w_down, residual, then)
-        gate_up = torch.empty((T, 2 * inter), dtype=torch.float32, device=ctx.device)
-        linear(h, self.w_gate_up, gate_up)
-        mid = torch.empty((T, inter), dtype=self.mid_dtype, device=ctx.device)
-        ops.silu_mul(gate_up, mid)
+        else:
+            gate_up = torch.empty((T, 2 * inter), dtype=torch.float32, device=ctx.device)
+            linear(h, self.w_gate_up, gate_up)
+            mid = torch.empty((T, inter), dtype=self.mid_dtype, device=ctx.device)
+            ops.act_mul(gate_up, mid, self.activation)
+        if overwrite:
+            linear(mid, self.w_down, residual)
+            return None
         return linear_onto(mid, self.w_down, residual, then)
 
 

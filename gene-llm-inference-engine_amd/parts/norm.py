@@ -76,6 +76,10 @@ class RmsNorm(Norm):
             x, rows = ops.gather_rows(x, rows, torch.empty((n, x.shape[1]), dtype=torch.float32, device=x.device)), None
         return ops.rmsnorm(x, self.weight, self.eps, out, rows)
 
+    def add_onto(self, y, x):
+        """x += norm(y), both float32 [T, size]: what a layer does whose norm follows a sublayer."""
+        return ops.rmsnorm_add(y, self.weight, self.eps, x)
+
     def deferred(self, x, out_dtype, rows=None) -> NormedRows:
         return NormedRows(self, x, out_dtype, rows)
 

@@ -40,4 +40,38 @@ class RotaryHalfSplit(PositionEncoding):
         return ctx.memo[key]
 
 
+class RotaryPartial(PositionEncoding):
+    """The same rotation on the first `rotary_dim` channels of a head only: pairs (i, i + rotary_dim/2); the rest of the head
+    passes.  It has no tables for whole heads; a mixer whose kernels turn a part of a head asks `partial_tables`."""
+    graph_safe = True
+
+    def __init__(self, spec, tensors, dtype, device):
+        super().__init__(spec, tensors, dtype, device)
+        self.rotary_dim = spec.rotary_dim
+        frequencies = spec.frequencies if spec.frequencies is not None else inverse_frequencies(spec.rotary_dim, spec.theta)
+        self.inv_freq = torch.tensor(list(frequencies), dtype=torch.float64, device=device)
+
+    def partial_tables(self, ctx):
+        """(cos, sin, rotary_dim): float32 [T, rotary_dim/2] each, for the rows of this step."""
+        key = ("rotary_partial", self.spec)
+        if key not in ctx.memo:
+            cos = torch.empty((ctx.n_rows, self.rotary_dim // 2), dtype=torch.float32, device=ctx.device)
+            sin = torch.empty_like(cos)
+            ops.rope_cos_sin(ctx.row_pos, self.inv_freq, cos, sin)
+            ctx.memo[key] = (cos, sin)
+        return (*ctx.memo[key], self.rotary_dim)
+
+
+def rotation_tables(position, ctx):
+    """(cos, sin, channels turned) of an encoding that turns the pairs (i, i + r/2) of a head's first r channels (the whole head
+    or a part), or None if `position` is no such encoding."""
+    if position is None:
+        return None
+    if hasattr(position, "partial_tables"):
+        return position.partial_tables(ctx)
+    tables = position.half_split_tables(ctx)
+    return None if tables is None else (*tables, 2 * tables[0].shape[1])
+
+
 register_position_encoding("rotary_half_split", RotaryHalfSplit)
+register_position_encoding("rotary_partial", RotaryPartial)
