@@ -418,7 +418,8 @@ class CacheManager:
             raise CacheError("a request with fixed-size state cannot be rewound: the state of earlier positions is gone")
         for g in self.groups:
             if not g.can_rewind_to(slot, length):
-                raise CacheError(f"request {request!r} cannot be rewound to {length}: a window or a chunk's end has given those pages back")
+                gone = f"a window of {g.need.window}" if g.need.window is not None else f"the end of a chunk of {g.need.chunk}"
+                raise CacheError(f"request {request!r} cannot be rewound to {length}: {gone} has given those pages back")
         for g in self.groups:
             if g.shared_page_at(slot, length) and g.pool.free_count + g.pages_freed_by_rewind(slot, length) < 1 and self.evict(1) < 1:
                 raise OutOfPages("no free page to copy a shared page into")
