@@ -26,6 +26,33 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) { return f32x2_to_bf
 constexpr float LOG2E = 1.4426950408889634f;
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// What a layer may ask for beyond causal attention with a window (all absent for a plain layer: 0 and null):
+//   chunk   a row at position p sees no key before p - p % chunk (a mask cut into chunks counted from the sequence's start);
+//   sinks   [n_heads]: exp(sinks[h]) joins the softmax's denominator of head h (a score without a key or a value), once a row:
+//           where a row's keys are shared out over splits or waves, the first of them counts it;
+//   gate    [rows, gate_stride]: head h's output of row t is multiplied by sigmoid(gate[t * gate_stride + h]).
+struct Extras {
+    int chunk;
+    const float* sinks;
+    const float* gate;
+    long gate_stride;
+};
+// The first position a row at `p` sees.
+__device__ __forceinline__ int lowest_seen(int p, int window, int chunk) {
+    int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    if (chunk > 0 && p > 0) lo = max(lo, p - p % chunk);
+    return lo;
+}
+// The sink joins {m, l} (m in units of log2 e).
+__device__ __forceinline__ void add_sink(float sink, float& m, float& l) {
+    const float s2 = sink * LOG2E;
+    if (m == -INFINITY) { m = s2; l = 1.f; }
+    else l += exp2_fast(s2 - m);
+}
+__device__ __forceinline__ float gate_of(const Extras& x, size_t row, int head) {
+    return x.gate ? 1.0f / (1.0f + expf(-x.gate[row * x.gate_stride + head])) : 1.0f;
+}
+
 // =========================================================================================== prompt
 // Workgroup: PAIR row tiles of one request (up to 32 * NW consecutive rows each), one query head.
 // 32 rows belong to two waves: each takes one half (32 positions) of every tile of 64 keys and
@@ -56,7 +83,8 @@ __global__ __launch_bounds__(128 * NW * PAIR) void attention_prompt_kernel(const
                                                                           bf16_t* __restrict__ out, const int4* __restrict__ tiles,
                                                                           const int* __restrict__ table, int table_stride, long page_stride,
                                                                           int page_size, int n_heads, int n_kv, int window, float scale,
-                                                                          int n_splits, const int* __restrict__ tile_first, float* __restrict__ part) {
+                                                                          int n_splits, const int* __restrict__ tile_first, float* __restrict__ part,
+                                                                          Extras extra) {
     constexpr int NT = 128 * NW * PAIR;         // threads
     constexpr int K_STRIDE = HD + 8;            // bf16 elements; 16-byte reads of 32 rows hit distinct banks
     constexpr int V_STRIDE = KV_TILE + 4;       // 8-byte reads of 32 rows hit distinct banks
@@ -87,13 +115,13 @@ __global__ __launch_bounds__(128 * NW * PAIR) void attention_prompt_kernel(const
     const int my_row = wv * 32 + col;                           // this lane's query row within its tile
     const bool row_ok = my_row < n_rows;
     const int my_pos = row_ok ? pos0 + my_row : -1;
-    const int my_lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
+    const int my_lo = lowest_seen(my_pos, window, extra.chunk);
     const int wave_last = pos0 + min(n_rows, wv * 32 + 32) - 1;         // the last position this wave's rows see
     const bool wave_ok = wv * 32 < n_rows;
     const bool wave_full = wv * 32 + 32 <= n_rows;
     const int wave_first = wave_full ? pos0 + wv * 32 : -1;             // keys up to here are seen by every row of the wave (none if rows are missing)
-    const int wave_lo_max = window > 0 ? max(0, wave_last - window + 1) : 0;      // ... and keys from here on
-    const int wave_lo_min = window > 0 ? max(0, pos0 + wv * 32 - window + 1) : 0; // no row of the wave sees a key before this one
+    const int wave_lo_max = lowest_seen(wave_last, window, extra.chunk);      // ... and keys from here on
+    const int wave_lo_min = lowest_seen(pos0 + wv * 32, window, extra.chunk); // no row of the wave sees a key before this one
     const float scale2 = scale * LOG2E;
 
     bf16x8 qreg[QSTEPS];
@@ -109,7 +137,7 @@ __global__ __launch_bounds__(128 * NW * PAIR) void attention_prompt_kernel(const
     float m = -INFINITY, l = 0.f;               // l: this lane's share of the sum (its partner lane^32 holds the rest)
 
     // the keys the workgroup walks: from the first one any of its rows sees to the last
-    auto lowest = [&](const int4 t) { return (window > 0 && t.z - window + 1 > 0) ? t.z - window + 1 : 0; };
+    auto lowest = [&](const int4 t) { return lowest_seen(t.z, window, extra.chunk); };
     int last_pos = tile_a.z + tile_a.y - 1, first_lo = lowest(tile_a);
     if (PAIR == 2 && tile_b.y > 0) {
         last_pos = max(last_pos, tile_b.z + tile_b.y - 1);
@@ -308,6 +336,7 @@ __global__ __launch_bounds__(128 * NW * PAIR) void attention_prompt_kernel(const
         }
     }
     if (!row_ok || ks != 0) return;
+    if (extra.sinks != nullptr && split == 0) add_sink(extra.sinks[head], m, l);
     if (n_splits > 1) {                                       // part[row of the split tiles][head][split] = {m, l, O[HD]}
         float* dst = part + (((size_t)(tile_first[PAIR * group + half] + my_row) * n_heads + head) * n_splits + split) * (HD + 2);
         if (hf == 0) {
@@ -320,7 +349,7 @@ __global__ __launch_bounds__(128 * NW * PAIR) void attention_prompt_kernel(const
             for (int v = 0; v < 16; ++v) dst[2 + 32 * i + 8 * (v / 4) + 4 * hf + (v & 3)] = o[i][v];
         return;
     }
-    const float inv = 1.0f / l;
+    const float inv = gate_of(extra, (size_t)(row0 + my_row), head) / l;
     bf16_t* orow = out + ((size_t)(row0 + my_row) * n_heads + head) * HD;
 #pragma unroll
     for (int i = 0; i < DT; ++i)
@@ -359,7 +388,7 @@ __global__ __launch_bounds__(64 * NW, HD == 128 ? 2 : 3) void attention_prompt_w
                                                                        const int* __restrict__ table, int table_stride, long page_stride,
                                                                        int page_size, int n_heads, int n_kv, int window, float scale,
                                                                        int n_splits, const int* __restrict__ tile_first, float* __restrict__ part,
-                                                                       int list_order) {
+                                                                       int list_order, Extras extra) {
     static_assert(HD == 128 || HD == 64, "the chunk swizzle is made for key rows of 256 or 128 bytes");
     constexpr int QSTEPS = HD / 16, DT = HD / 32;
     constexpr int K_BYTES = KV_TILE * HD * 2, V_BYTES = HD * KV_TILE * 2, STAGE = K_BYTES + V_BYTES;
@@ -386,13 +415,13 @@ __global__ __launch_bounds__(64 * NW, HD == 128 ? 2 : 3) void attention_prompt_w
     const int my_row = wv * 32 + col;
     const bool row_ok = my_row < n_rows;
     const int my_pos = row_ok ? pos0 + my_row : -1;
-    const int my_lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
+    const int my_lo = lowest_seen(my_pos, window, extra.chunk);
     const int wave_last = pos0 + min(n_rows, wv * 32 + 32) - 1;
     const bool wave_ok = wv * 32 < n_rows;
     const bool wave_full = wv * 32 + 32 <= n_rows;
     const int wave_first = wave_full ? pos0 + wv * 32 : -1;
-    const int wave_lo_max = window > 0 ? max(0, wave_last - window + 1) : 0;
-    const int wave_lo_min = window > 0 ? max(0, pos0 + wv * 32 - window + 1) : 0;
+    const int wave_lo_max = lowest_seen(wave_last, window, extra.chunk);
+    const int wave_lo_min = lowest_seen(pos0 + wv * 32, window, extra.chunk);
     const float scale2 = scale * LOG2E;
 
     bf16x8 qreg[QSTEPS];
@@ -408,7 +437,7 @@ __global__ __launch_bounds__(64 * NW, HD == 128 ? 2 : 3) void attention_prompt_w
     float m = -INFINITY, l = 0.f;
 
     const int last_pos = pos0 + n_rows - 1;
-    const int first_lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+    const int first_lo = lowest_seen(pos0, window, extra.chunk);
     const int range_first = first_lo & ~(KV_TILE - 1);
     const int per_split = ((last_pos - range_first) / KV_TILE + n_splits) / n_splits * KV_TILE;
     const int kv_first = range_first + split * per_split, my_last = min(last_pos, kv_first + per_split - 1);
@@ -549,6 +578,7 @@ __global__ __launch_bounds__(64 * NW, HD == 128 ? 2 : 3) void attention_prompt_w
     }
     l += __shfl_xor(l, 32, 64);
     if (!row_ok) return;
+    if (extra.sinks != nullptr && split == 0) add_sink(extra.sinks[head], m, l);
     if (n_splits > 1) {                                       // part[row of the split tiles][head][split] = {m, l, O[HD]}
         float* dst = part + (((size_t)(tile_first[group] + my_row) * n_heads + head) * n_splits + split) * (HD + 2);
         if (hf == 0) {
@@ -561,7 +591,7 @@ __global__ __launch_bounds__(64 * NW, HD == 128 ? 2 : 3) void attention_prompt_w
             for (int v = 0; v < 16; ++v) dst[2 + 32 * i + 8 * (v / 4) + 4 * hf + (v & 3)] = o[i][v];
         return;
     }
-    const float inv = 1.0f / l;
+    const float inv = gate_of(extra, (size_t)(row0 + my_row), head) / l;
     bf16_t* orow = out + ((size_t)(row0 + my_row) * n_heads + head) * HD;
 #pragma unroll
     for (int i = 0; i < DT; ++i)
@@ -641,7 +671,7 @@ __global__ __launch_bounds__(64 * DecodeShape<HD>::MAX_WAVES) void attention_dec
     long ldv, const float* __restrict__ cos_t, const float* __restrict__ sin_t, bf16_t* __restrict__ cache, float* __restrict__ part,
     bf16_t* __restrict__ out, const int* __restrict__ rows, const int* __restrict__ pos, const int* __restrict__ slots,
     const int* __restrict__ table, int table_stride, long page_stride, int page_size, int n_heads, int n_kv, int window, float scale,
-    int n_splits, int gh) {
+    int n_splits, int gh, Extras extra) {
     constexpr int KSTEPS = HD / 32, DT = HD / 16;
     extern __shared__ float merged[];                        // [wave][gh][HD + 2]
     const int group = n_heads / n_kv, hg_per_kv = (group + 15) / 16;
@@ -669,7 +699,7 @@ __global__ __launch_bounds__(64 * DecodeShape<HD>::MAX_WAVES) void attention_dec
         for (int s = 0; s < KSTEPS; ++s) q_raw[s] = load_pairs8(qf + (size_t)row * ldq + (size_t)(head_ok ? head : g * group) * HD, 32 * s + 8 * q4, HD / 2);
     }
     const int my_pos = pos[row];
-    const int lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
+    const int lo = lowest_seen(my_pos, window, extra.chunk);
     const int* tab = table + (size_t)__builtin_amdgcn_readfirstlane(slots[row]) * table_stride;
     // every row cuts its own range into pieces (multiples of 32), one per wave of every split; short rows leave later pieces empty
     const int n_pieces = n_splits * n_waves, piece = split * n_waves + wave;
@@ -899,8 +929,9 @@ __global__ __launch_bounds__(64 * DecodeShape<HD>::MAX_WAVES) void attention_dec
             denom = fmaf(weight, first[w * wave_stride + 1], denom);
             acc = fmaf(weight, first[w * wave_stride + 2 + d], acc);
         }
+        if (extra.sinks != nullptr && split == 0) add_sink(extra.sinks[out_head], big, denom);
         if (n_splits == 1) {
-            out[((size_t)row * n_heads + out_head) * HD + d] = f32_to_bf16(acc / denom);
+            out[((size_t)row * n_heads + out_head) * HD + d] = f32_to_bf16(acc / denom * gate_of(extra, (size_t)row, out_head));
         } else {                                             // part[row_index][head][split] = {m, l, O[HD]}
             float* dst = part + (((size_t)blockIdx.x * n_heads + out_head) * n_splits + split) * (HD + 2);
             if (d == 0) {
@@ -918,7 +949,7 @@ __global__ __launch_bounds__(64 * DecodeShape<HD>::MAX_WAVES) void attention_dec
 constexpr int MAX_SPLITS = 256;
 
 __global__ __launch_bounds__(64) void attention_decode_combine_kernel(const float* __restrict__ part, bf16_t* __restrict__ out,
-                                                                     const int* __restrict__ rows, int n_heads, int hd, int n_splits) {
+                                                                     const int* __restrict__ rows, int n_heads, int hd, int n_splits, Extras extra) {
     __shared__ float weight[MAX_SPLITS], weighted_l[MAX_SPLITS];
     constexpr int EARLY = 8;                                 // splits whose channels are asked for together with the splits' {m, l}
     const int idx = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
@@ -956,7 +987,7 @@ __global__ __launch_bounds__(64) void attention_decode_combine_kernel(const floa
     __syncthreads();
     float denom = 0.f;
     for (int s = 0; s < n_splits; ++s) denom += weighted_l[s];
-    const float inv = 1.0f / denom;
+    const float inv = gate_of(extra, (size_t)(rows ? rows[idx] : idx), head) / denom;
     const int n_early = min(n_splits, EARLY);
     for (int d = lane, c = 0; d < hd; d += 64, ++c) {
         float acc = 0.f;
@@ -987,7 +1018,9 @@ GI_API int gi_attention_bf16_supports(int hd, int page_size, int prompt) {
 GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out, const int* tiles, int n_tiles, int rows_per_tile, int paired,
                                     const int* table, int table_stride, long page_stride, int page_size, int n_heads, int n_kv, int hd,
                                     int window, float scale, int n_splits, const int* tile_first, const int* rows, int n_rows, float* part,
-                                    long part_floats, hipStream_t stream) {
+                                    long part_floats, int chunk, const float* sinks, const float* gate, long gate_stride, hipStream_t stream) {
+    GI_REQUIRE(chunk >= 0 && (gate == nullptr || gate_stride >= n_heads), "attention_prompt: bad chunk or gate stride");
+    const Extras extra = {chunk, sinks, gate, gate_stride};
     GI_REQUIRE(rows_per_tile == 64 || rows_per_tile == 128, "attention_prompt: tiles of %d rows are not supported (64 or 128)", rows_per_tile);
     GI_REQUIRE(n_tiles > 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attention_prompt: bad counts (%d tiles, %d heads, %d kv heads)",
                n_tiles, n_heads, n_kv);
@@ -1011,14 +1044,14 @@ GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out,
 #define WIDE(HD, NW)                                                                                                                    \
     attention_prompt_wide_kernel<HD, NW><<<wgrid, 64 * NW, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, (bf16_t*)out, (const int4*)tiles, table, \
                                                                        table_stride, page_stride, page_size, n_heads, n_kv, window, scale, n_splits, \
-                                                                       tile_first, part, paired ? 1 : 0)
+                                                                       tile_first, part, paired ? 1 : 0, extra)
         if (hd == 64) { if (rows_per_tile == 64) WIDE(64, 2); else WIDE(64, 4); }
         else WIDE(128, 4);      // (tiles of 64 rows too: two of its waves then only load; a workgroup of two waves would need 16 loads a wave and more registers than two to a SIMD leave)
 #undef WIDE
         GI_CHECK_LAUNCH("attention_prompt (wide)");
         if (n_splits > 1) {
             dim3 cgrid(n_rows, n_heads);
-            attention_decode_combine_kernel<<<cgrid, 64, 0, stream>>>(part, (bf16_t*)out, rows, n_heads, hd, n_splits);
+            attention_decode_combine_kernel<<<cgrid, 64, 0, stream>>>(part, (bf16_t*)out, rows, n_heads, hd, n_splits, extra);
             GI_CHECK_LAUNCH("attention_prompt (combine)");
         }
         return 0;
@@ -1028,7 +1061,7 @@ GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out,
 #define GO_(HD, NW, PAIR)                                                                                                               \
     attention_prompt_kernel<HD, NW, PAIR><<<grid, 128 * NW * PAIR, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, (bf16_t*)out, (const int4*)tiles, \
                                                                                 table, table_stride, page_stride, page_size, n_heads, n_kv, window, \
-                                                                                scale, n_splits, tile_first, part)
+                                                                                scale, n_splits, tile_first, part, extra)
 #define GO(HD)                                                                                                                          \
     do {                                                                                                                                \
         if (rows_per_tile == 64) { if (pairs) GO_(HD, 2, (HD <= 64 ? 2 : 1)); else GO_(HD, 2, 1); }                                     \
@@ -1040,7 +1073,7 @@ GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out,
     GI_CHECK_LAUNCH("attention_prompt");
     if (n_splits > 1) {
         dim3 cgrid(n_rows, n_heads);
-        attention_decode_combine_kernel<<<cgrid, 64, 0, stream>>>(part, (bf16_t*)out, rows, n_heads, hd, n_splits);
+        attention_decode_combine_kernel<<<cgrid, 64, 0, stream>>>(part, (bf16_t*)out, rows, n_heads, hd, n_splits, extra);
         GI_CHECK_LAUNCH("attention_prompt (combine)");
     }
     return 0;
@@ -1089,7 +1122,9 @@ GI_API int gi_attention_decode_bf16(const void* q, const float* qf, const float*
                                     const float* cos_t, const float* sin_t, void* cache, void* out, float* part, long part_floats,
                                     const int* rows, int n_rows, const int* pos, const int* slots, const int* table, int table_stride,
                                     long page_stride, int page_size, int n_heads, int n_kv, int hd, int window, float scale, int n_splits,
-                                    int n_waves, hipStream_t stream) {
+                                    int n_waves, int chunk, const float* sinks, const float* gate, long gate_stride, hipStream_t stream) {
+    GI_REQUIRE(chunk >= 0 && (gate == nullptr || gate_stride >= n_heads), "attention_decode: bad chunk or gate stride");
+    const Extras extra = {chunk, sinks, gate, gate_stride};
     GI_REQUIRE(n_rows > 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attention_decode: bad counts (%d rows, %d heads, %d kv heads)",
                n_rows, n_heads, n_kv);
     GI_REQUIRE(gi_attention_bf16_supports(hd, page_size, 0), "attention_decode: head size %d with page size %d is not supported", hd, page_size);
@@ -1121,7 +1156,7 @@ GI_API int gi_attention_decode_bf16(const void* q, const float* qf, const float*
     attention_decode_kernel<HD, FUSED_><<<grid, 64 * n_waves, lds, stream>>>((const bf16_t*)q, qf, kf, vf, ldq, ldk, ldv, cos_t, sin_t,   \
                                                                              (bf16_t*)cache, part, (bf16_t*)out, rows, pos, slots, table, \
                                                                              table_stride, page_stride, page_size, n_heads, n_kv, window,  \
-                                                                             scale, n_splits, gh)
+                                                                             scale, n_splits, gh, extra)
 #define GO(HD)                    \
     do {                          \
         if (qf) GO2(HD, true);    \
@@ -1133,7 +1168,7 @@ GI_API int gi_attention_decode_bf16(const void* q, const float* qf, const float*
     GI_CHECK_LAUNCH("attention_decode");
     if (n_splits > 1) {
         dim3 cgrid(n_rows, n_heads);
-        attention_decode_combine_kernel<<<cgrid, 64, 0, stream>>>(part, (bf16_t*)out, rows, n_heads, hd, n_splits);
+        attention_decode_combine_kernel<<<cgrid, 64, 0, stream>>>(part, (bf16_t*)out, rows, n_heads, hd, n_splits, extra);
         GI_CHECK_LAUNCH("attention_decode (combine)");
     }
     return 0;

@@ -46,10 +46,10 @@ _SIGNATURES = {
     "gi_head_norm_gate": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_float, c_void_p],
     "gi_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long, c_void_p],
     "gi_attention_prompt_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
-                                 c_float, c_int, c_void_p, c_void_p, c_int, c_void_p, c_long, c_void_p],
+                                 c_float, c_int, c_void_p, c_void_p, c_int, c_void_p, c_long, c_int, c_void_p, c_void_p, c_long, c_void_p],
     "gi_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_long, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_long, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
-                                 c_float, c_int, c_int, c_void_p],
+                                 c_float, c_int, c_int, c_int, c_void_p, c_void_p, c_long, c_void_p],
     "gi_random_normal": [c_void_p, c_int, c_long, ctypes.c_ulonglong, ctypes.c_double, ctypes.c_double, c_void_p],
     "gi_probe_stream": [c_void_p, c_void_p, c_long, c_void_p, c_int, c_int, c_void_p],
     "gi_probe_mfma": [c_int, c_void_p, c_int, c_void_p],
@@ -772,15 +772,25 @@ def decode_attention_shape(n_decode, n_heads, n_kv, hd, span, target_waves=4096,
 
 
 def attention_bf16(q, cache, out, plan: AttentionPlan, positions, slots, table, n_heads, n_kv, hd, window=None, scale=None,
-                   target_waves: int = 4096, products=None):
+                   target_waves: int = 4096, products=None, chunk=None, sinks=None, gate=None):
     """Attention of a step's rows with the matrix-core kernels (bfloat16 cache and out).
 
     `q` holds the rotated queries in bfloat16 and the cache the rows' keys and values; or, for a step
     of single decoded rows only, `q` is None and `products = (q, k, v, cos, sin)` holds the unrotated
     float32 products and the rotation's tables (k, v None: the pages are another layer's; cos, sin
-    None: no rotation): the decode kernel then rotates, writes the cache and attends in one launch."""
+    None: no rotation): the decode kernel then rotates, writes the cache and attends in one launch.
+
+    chunk, sinks, gate: as `attention_exact` takes them (a mask cut into chunks, a score per head that joins the softmax's
+    denominator only, a gate per row and head on the output)."""
     n = out.shape[0]
-    _dev(q, cache, out, positions, slots, table)
+    _dev(q, cache, out, positions, slots, table, sinks, gate)
+    if sinks is not None and not (sinks.dtype == torch.float32 and sinks.is_contiguous() and sinks.numel() == n_heads):
+        raise KernelError("attention: sinks must be float32 [heads]")
+    if gate is not None and not (gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape[0] == n and gate.shape[1] >= n_heads and gate.stride(1) == 1):
+        raise KernelError("attention: the heads' gates must be float32 [n, heads] with unit inner stride")
+    chunk = int(chunk or 0)
+    extras = (chunk, _ptr(sinks), _ptr(gate), gate.stride(0) if gate is not None else 0)
+    seen = lambda context, slack: min([context] + ([window + slack] if window else []) + ([chunk + slack] if chunk else []))
     for t, name in ((q, "q"), (cache, "cache"), (out, "out")):
         if not (t is None or t.dtype == torch.bfloat16):
             raise KernelError(f"attention_bf16: {name} must be bfloat16")
@@ -809,23 +819,22 @@ def attention_bf16(q, cache, out, plan: AttentionPlan, positions, slots, table, 
             if not (t is None or (t.dtype == torch.float32 and t.shape == (n, hd // 2) and t.is_contiguous())):
                 raise KernelError("attention: cos/sin must be float32 [n, hd/2]")
     if plan.n_tiles:
-        n_splits = prompt_attention_splits(plan.n_tiles // 2 if plan.paired else plan.n_tiles, n_heads,
-                                           plan.max_tile_context if not window else min(plan.max_tile_context, window + plan.tile),
+        n_splits = prompt_attention_splits(plan.n_tiles // 2 if plan.paired else plan.n_tiles, n_heads, seen(plan.max_tile_context, plan.tile),
                                            target_groups=PAIRED_TARGET_GROUPS if plan.paired else 512)      # a pair's workgroup has twice the waves
         n_part = plan.n_tile_rows * n_heads * n_splits * (hd + 2) if n_splits > 1 else 0
         part = torch.empty(n_part, dtype=torch.float32, device=out.device) if n_part else None
         _call("gi_attention_prompt_bf16", q.data_ptr(), cache.data_ptr(), out.data_ptr(), plan.tiles.data_ptr(), plan.n_tiles, plan.tile,
               1 if plan.paired else 0, table.data_ptr(), table.stride(0), cache.stride(0), page_size, n_heads, n_kv, hd, window, scale, n_splits,
-              _ptr(plan.tile_first), _ptr(plan.tile_rows), plan.n_tile_rows, _ptr(part), n_part, _stream())
+              _ptr(plan.tile_first), _ptr(plan.tile_rows), plan.n_tile_rows, _ptr(part), n_part, *extras, _stream())
     if plan.n_decode:
-        span = plan.max_decode_context if not window else min(plan.max_decode_context, window + 31)
+        span = seen(plan.max_decode_context, 31)
         n_splits, n_waves = decode_attention_shape(plan.n_decode, n_heads, n_kv, hd, span, target_waves, products is not None)
         n_part = plan.n_decode * n_heads * n_splits * (hd + 2) if n_splits > 1 else 0
         part = torch.empty(n_part, dtype=torch.float32, device=out.device) if n_part else None
         _call("gi_attention_decode_bf16", _ptr(q), _ptr(qf), _ptr(kf), _ptr(vf), qf.stride(0) if qf is not None else 0,
               kf.stride(0) if kf is not None else 0, vf.stride(0) if vf is not None else 0, _ptr(cos), _ptr(sin), cache.data_ptr(),
               out.data_ptr(), _ptr(part), n_part, _ptr(plan.decode_rows), plan.n_decode, positions.data_ptr(), slots.data_ptr(),
-              table.data_ptr(), table.stride(0), cache.stride(0), page_size, n_heads, n_kv, hd, window, scale, n_splits, n_waves, _stream())
+              table.data_ptr(), table.stride(0), cache.stride(0), page_size, n_heads, n_kv, hd, window, scale, n_splits, n_waves, *extras, _stream())
     return out
 
 
@@ -848,6 +857,12 @@ def attention(q, cache, out, ctx, table, n_heads, n_kv, hd, window=None):
 def attention_general(q, cache, out, ctx, table, n_heads, n_kv, hd, *, page_size, value_dim=None, window=None, chunk=None, scale=None, sinks=None, gate=None):
     """Attention of a step's rows for layers with any of: value heads of another size, a scale of their own, a mask cut into
     chunks, sinks, a gate per head."""
+    vd = int(value_dim or hd)
+    if (vd == hd and cache.dim() == 5 and q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
+            and (gate is None or gate.dtype == torch.float32)):
+        plan = _plan_of(ctx)
+        if (not plan.n_tiles or attention_bf16_supports(hd, page_size, True)) and (not plan.n_decode or attention_bf16_supports(hd, page_size, False)):
+            return attention_bf16(q, cache, out, plan, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window, scale, chunk=chunk, sinks=sinks, gate=gate)
     return attention_exact(q, cache, out, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window, scale, page_size=page_size,
                            value_dim=value_dim, chunk=chunk, sinks=sinks, gate=gate)
 

@@ -340,3 +340,32 @@ def test_greedy_generation_through_the_entry_point_and_the_scheduler(folders):
     ids = [eng.submit(EngineRequest(p, len(p) + 7, SamplerConfig(0.0))) for p in prompts]
     eng.run_until_idle()
     assert [eng.result(i).generated_tokens for i in ids] == want
+
+
+@pytest.mark.parametrize("hd, heads, kv, chunk", [(64, 4, 2, 64), (64, 6, 1, 80), (128, 4, 4, 200), (32, 2, 1, 48), (64, 32, 8, 1000), (64, 2, 1, 2000)])
+def test_matrix_core_attention_with_chunks_sinks_and_gates(hd, heads, kv, chunk):
+    """The bfloat16 kernels on the matrix cores against the 32-bit-arithmetic kernel on the same pages and queries: a long
+    portion on top of a past (tiles, pairs of tiles, keys shared out), short portions and single rows of other requests."""
+    from geneinfer_amd.kernels import ops
+    from geneinfer_amd.parts import StepContext
+    g = torch.Generator().manual_seed(hd + chunk)
+    page, scale = 16, 0.7 * hd ** -0.5
+    lens, pos0 = [300, 1, 40, 1, 700], [150, 333, 90, 0, 0]
+    n_slots, width = len(lens), -(-1100 // page)
+    table = torch.randperm(n_slots * width, generator=g).to(torch.int32).view(n_slots, width)
+    cache = (torch.randn(n_slots * width, 2, kv, page, hd, generator=g)).to(torch.bfloat16).to(DEV)
+    T = sum(lens)
+    starts = [sum(lens[:i]) for i in range(n_slots)]
+    q = torch.randn(T, heads * hd, generator=g).to(torch.bfloat16).to(DEV)
+    pos = torch.tensor([p + i for p, n in zip(pos0, lens) for i in range(n)], dtype=torch.int32, device=DEV)
+    slot = torch.tensor([s for s, n in enumerate(lens) for _ in range(n)], dtype=torch.int32, device=DEV)
+    sinks = (2 * torch.randn(heads, generator=g)).to(DEV)
+    gate = torch.randn(T, heads + 3, generator=g).to(DEV)[:, :heads]
+    ctx = StepContext(n_rows=T, dtype=torch.bfloat16, device=torch.device(DEV), tokens=slot, row_pos=pos, row_slot=slot, seg_slot=list(range(n_slots)),
+                      seg_start=starts, seg_len=lens, seg_pos0=pos0)
+    for extras in (dict(chunk=chunk, sinks=sinks, gate=gate), dict(chunk=chunk), dict(sinks=sinks), dict(gate=gate)):
+        fast = ops.attention_general(q, cache, torch.empty_like(q), ctx, table.to(DEV), heads, kv, hd, page_size=page, scale=scale, **extras)
+        slow = ops.attention_exact(q, cache, torch.empty_like(q), pos, slot, table.to(DEV), heads, kv, hd, None, scale, **extras)
+        assert relative_error(fast.float(), slow.float()) < 2e-2, sorted(extras)
+        worst = (fast.float() - slow.float()).abs().view(T, heads, hd).amax(dim=(1, 2))
+        assert float(worst.max()) < 0.06, (sorted(extras), int(worst.argmax()))
