@@ -1,6 +1,7 @@
 """Decode and prefill throughput of the engine at the Llama-3.2-1B shape, random weights, one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--config FILE] [--prefill-tokens T] [--layers L] [--no-points]
+    python bench.py --fekorax [--sizes 1b,8b] [--layers L] [--batch B] [--prefill-tokens T]     (another record: see `fekorax_beside_llama`)
 
 A step is one decode step of the whole batch (default batch 8, each request on a 2,048-token
 prompt in a 4,096-token context), through the scheduler with its defaults.  After W warm-up steps,
@@ -35,6 +36,91 @@ LLAMA_1B = dict(hidden_size=2048, intermediate_size=8192, num_hidden_layers=16, 
 PROMPT, NEW_TOKENS, CONTEXT, PAGE = 2048, 256, 4096, 16
 
 
+# Layer shapes for `--fekorax`: (hidden, heads, key/value heads, head size, feed-forward's inner size, vocabulary).
+FEKORAX_SIZES = {"1b": (2048, 32, 8, 64, 8192, 32000), "3b": (3072, 24, 8, 128, 8192, 32000), "8b": (4096, 32, 8, 128, 14336, 32000)}
+
+
+def fekorax_beside_llama(args) -> int:
+    """The Fekorax design at layer shapes of real models beside the Llama decoder at the same shapes, random weights: prefill of one
+    prompt and decode steps of a batch on that context, through the step function (captured decode steps), and the time of every
+    kernel in both (the device waited for around each).  A Fekorax model of L layers here is L/4 times [matrix memory; attention +
+    feed-forward; matrix memory; attention on the pages of the one before + feed-forward], the attention with the Llama layer's
+    heads (rotation of half of each head, chunks of 1,024, sinks, head gates), the matrix memories with a quarter as many heads of
+    the same key size and twice the value size; the Llama model has L layers of attention + feed-forward.  One JSON line."""
+    import torch
+    from geneinfer_amd.config import parse_config
+    from geneinfer_amd.engine import Runner, StepEntry, random_model
+    from geneinfer_amd.kernels import ops
+
+    T, batch, L, steps = args.prefill_tokens, args.batch, args.layers or 8, args.steps
+    gen = torch.Generator().manual_seed(1)
+    record = {"metric": "Fekorax beside Llama at equal layer shapes: prefill tok/s, decode ms a step, ms by kernel", "dtype": args.dtype, "layers": L,
+              "prefill_tokens": T, "decode_batch": batch, "data": "synthetic: random weights by formula, uniform random token ids", "sizes": {}}
+    for size in args.sizes.split(","):
+        D, H, G, hd, ff, vocab = FEKORAX_SIZES[size]
+        llama = dict(architectures=["LlamaForCausalLM"], hidden_size=D, intermediate_size=ff, num_hidden_layers=L, num_attention_heads=H,
+                     num_key_value_heads=G, head_dim=hd, vocab_size=vocab, max_position_embeddings=T + 1024, rope_theta=500000.0, rms_norm_eps=1e-5,
+                     tie_word_embeddings=True)
+        att = lambda source=None: dict(type="attention", mlp=dict(kind="dense", ff=ff), mixer=dict(
+            heads=H, kv_heads=G, dim=hd, vdim=hd, scale=hd ** -0.5, rot=dict(dims=hd // 2, base=10000.0), mask=dict(size=1024),
+            **({} if source is None else dict(kv_from=source))))
+        mem = dict(type="mlstm", mlp=None, mixer=dict(heads=max(1, H // 4), dim=hd, vdim=2 * hd, gate_cap=15.0))
+        layers = []
+        for i in range(0, L, 4):
+            layers += [mem, att(), mem, att(i + 1)]
+        fekorax = dict(architecture="Fekorax", vocab=vocab, width=D, embedding=dict(scale=D ** 0.5), norm=dict(eps=1e-5), layers=layers[:L],
+                       max_positions=T + 1024)
+        record["sizes"][size] = {}
+        for name, cfg in (("llama", llama), ("fekorax", fekorax)):
+            model = random_model(parse_config(cfg), seed=0, dtype="bfloat16" if args.dtype == "bf16" else "float32", device="cuda:0", draw_on_device=True)
+            runner = Runner(model, page_size=PAGE, max_tokens=batch * (T + 512), max_requests=batch, max_rows=max(T, batch), max_positions=T + 1024)
+            prompts = [torch.randint(0, vocab, (T,), generator=gen).tolist() for _ in range(batch)]
+
+            def prefill_all():
+                times = []
+                for r, p in enumerate(prompts):
+                    if runner.is_open(r):
+                        runner.close(r)
+                    runner.open(r)
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    runner.step([StepEntry(r, p, (T - 1,))])
+                    torch.cuda.synchronize()
+                    times.append(time.perf_counter() - t0)
+                return sorted(times)[len(times) // 2]
+
+            def decode_steps(n):
+                entries = [StepEntry(r, [7], (0,)) for r in range(batch)]
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(n):
+                    runner.step(entries)
+                torch.cuda.synchronize()
+                return (time.perf_counter() - t0) / n
+
+            prefill_all()
+            prefill_s = prefill_all()
+            decode_steps(args.warmup)
+            decode_s = sorted(decode_steps(steps) for _ in range(3))[1]
+            # the same once more with every kernel timed (no captured steps meanwhile)
+            by_kernel = {}
+            for what, run in (("prefill", lambda: (runner.close(0), runner.open(0), runner.step([StepEntry(0, prompts[0], (T - 1,))]))),
+                              ("decode", lambda: decode_steps(4))):
+                profile = ops.set_profiling(True)
+                run()
+                torch.cuda.synchronize()
+                n = 1 if what == "prefill" else 4
+                by_kernel[what] = {k: [profile.calls[k] // n, round(v * 1e3 / n, 4)] for k, v in sorted(profile.seconds.items(), key=lambda kv: -kv[1])}
+                ops.set_profiling(False)
+            record["sizes"][size][name] = {"prefill_tok_s": round(T / prefill_s, 1), "prefill_ms": round(prefill_s * 1e3, 3), "decode_ms_per_step": round(decode_s * 1e3, 4),
+                                           "decode_tok_s": round(batch / decode_s, 1), "weight_bytes_per_step": model.weight_bytes_read_per_step(),
+                                           "kernels_calls_ms": by_kernel}
+            del runner, model
+            torch.cuda.empty_cache()
+    print(json.dumps(record))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -46,10 +132,15 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     ap.add_argument("--config", default="", help="a config.json of another size of the architecture (default: the Llama-3.2-1B shape)")
     ap.add_argument("--prefill-tokens", type=int, default=PROMPT, help="length of the timed prompt")
+    ap.add_argument("--fekorax", action="store_true", help="another measurement: the Fekorax design beside Llama at equal layer shapes (see fekorax_beside_llama)")
+    ap.add_argument("--sizes", default="1b,8b", help="with --fekorax: layer shapes, of " + ", ".join(FEKORAX_SIZES))
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine")
         return 2
+
+    if args.fekorax:
+        return fekorax_beside_llama(args)
 
     import torch
     from geneinfer_amd.config import LlamaConfig

@@ -6,14 +6,19 @@
 //     S_t = exp(f_t + m_(t-1) - m_t) S_(t-1) + exp(i_t - m_t) k_t v_t^T        n_t likewise with k_t alone
 //     o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6)
 // with i_t = cap * tanh(pre_i / cap) and f_t = logsigmoid(cap * tanh(pre_f / cap)); S, n and m are zero at a sequence's start
-// (m = 0, not minus infinity).  Columns of S never meet, so a workgroup owns 64 of them (a "tile") for one head of one
-// request and walks the request's rows of this step in order; it keeps its own copy of n and m, which every tile of the head
-// computes alike.  State of one request slot: [head][tile]{S tile [dk][64], n [dk, padded to 4], m, 3 unused}, 32-bit.
+// (m = 0, not minus infinity).  Columns of S never meet, so one wave owns C of them (a "tile": 16, 8 or 4, fewer for longer
+// keys) for one head of one request and walks the request's rows of this step in order; it keeps its own copy of n and m,
+// which every tile of the head computes alike.  State of one request slot: [head][tile]{S tile [dk][C], n [dk, padded to 4],
+// m, 3 unused}, 32-bit.
 //
-// Inside the workgroup wave r of 4 keeps rows r*ROWS .. r*ROWS+ROWS-1 of the tile in registers, lane j column j.  Per token:
-// k and q*scale come through LDS (read as broadcasts), the four waves' shares of S^T q and n . q are added through LDS by
-// wave 0, which writes the outputs; the next token's k, q and v are asked for before the current one is worked on.  One
-// barrier a token.  The gates of 64 tokens are made at once by wave 0.  Every sum's order is fixed by (dk, ROWS) alone.
+// Lane = (column, group of rows): a lane keeps ROWS rows (RG apart) of one column in registers, the 64/C groups' shares of S^T q and
+// n . q (neighbouring lanes) are added by the vector unit's lane moves, so a token costs no barrier and no trip through LDS
+// for the sums, and the chip gets heads * dv / C independent waves.
+// Per token k and q*scale come through LDS (read as broadcasts).  The k, q and v of a block of tokens are asked for while the
+// block before it is worked on and laid into LDS at its end, so that no token waits for memory.  The gates of 64 tokens are made
+// at once, lane by token: m runs along them one after the other (an addition and a maximum each), and the exponentials it needs
+// are then taken for all 64 at once.  Every sum's order is fixed by dk alone: a request's results have the same bits however
+// its rows are cut into steps.
 #include "common.h"
 
 namespace {
@@ -36,97 +41,172 @@ __global__ __launch_bounds__(64) void segments_kernel(const int* __restrict__ sl
     for (int s = lane; s < n_segs; s += 64) seg_len[s] = s < count ? ((s + 1 < count ? seg_start[s + 1] : n_rows) - seg_start[s]) : 0;
 }
 
+// Lane `u`'s value of x, u the same for every lane.
+__device__ __forceinline__ float lane_value(float x, int u) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), u)); }
+
+// Sum over each group of RG neighbouring lanes (4, 8 or 16: within a row of 16 lanes), by the data-parallel moves of the vector
+// unit: a lane and its mirror image in the group, then lanes two apart, then neighbours.  Every lane of a group ends with the
+// same bits (each level adds the same two numbers on both sides).
+template <int CTRL>
+__device__ __forceinline__ float dpp_moved(float x) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, false));
+}
+template <int RG>
+__device__ __forceinline__ float group_sum(float x) {
+    static_assert(RG == 4 || RG == 8 || RG == 16, "groups of 4, 8 or 16 lanes");
+    if constexpr (RG == 16) x += dpp_moved<0x140>(x);        // row_mirror: lane i <-> 15 - i
+    if constexpr (RG >= 8) x += dpp_moved<0x141>(x);         // row_half_mirror: lane i <-> 7 - i
+    x += dpp_moved<0x4E>(x);                                 // quad_perm [2, 3, 0, 1]
+    x += dpp_moved<0xB1>(x);                                 // quad_perm [1, 0, 3, 2]
+    return x;
+}
+
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
-template <int ROWS>
-__global__ __launch_bounds__(256) void mlstm_scan_kernel(const float* __restrict__ proj, long ld, int q_off, int k_off, int v_off, int i_off, int f_off,
-                                                        const float* __restrict__ i_bias, const float* __restrict__ f_bias, float cap, float q_scale,
-                                                        const int* __restrict__ seg_start, const int* __restrict__ seg_len,
-                                                        const int* __restrict__ row_slot, float* __restrict__ state, long state_stride,
-                                                        float* __restrict__ out, long ldo, int dk, int dv) {
-    __shared__ float2 kq_s[2][4 * ROWS];
-    __shared__ float red[2][4][64];
-    __shared__ float red_n[2][4];
-    __shared__ float gate_i[64], gate_f[64];
+template <int C, int ROWS>
+__global__ __launch_bounds__(64) void mlstm_scan_kernel(const float* __restrict__ proj, long ld, int q_off, int k_off, int v_off, int i_off, int f_off,
+                                                       const float* __restrict__ i_bias, const float* __restrict__ f_bias, float cap, float q_scale,
+                                                       const int* __restrict__ seg_start, const int* __restrict__ seg_len,
+                                                       const int* __restrict__ row_slot, float* __restrict__ state, long state_stride,
+                                                       float* __restrict__ out, long ldo, int dk, int dv) {
+    constexpr int RG = 64 / C;                   // groups of rows: lane = column * RG + group, so that a column's groups are neighbouring lanes
+    constexpr int KQ = RG * ROWS;                // rows a token's k and q cover (dk, padded with zeros)
+    constexpr int TB = 1024 / KQ;                // tokens staged at a time: their k, q and v wait in LDS while the block before them is worked on
+    constexpr int PER = TB * KQ / 64;            // (k, q) pairs a lane brings per block
+    static_assert(TB >= 2 && TB <= 64 && 64 % TB == 0, "staging blocks divide the gates' blocks of 64 tokens");
+    constexpr int VPER = (TB * C + 63) / 64;     // values a lane brings per block
+    __shared__ float2 kq_s[2][TB][KQ];
+    __shared__ float v_s[2][TB][C];
+    __shared__ float4 coef[64];                  // per token of the gates' block: {decay of what is held, weight of what comes, exp(-m), -}
     const int seg = blockIdx.x, h = blockIdx.y, vt = blockIdx.z, n_tiles = gridDim.z;
-    const int tid = threadIdx.x, r = tid >> 6, j = tid & 63;
+    const int lane = threadIdx.x, c = lane / RG, rg = lane % RG;
     const int n = seg_len[seg];
     if (n <= 0) return;
     const int t0 = seg_start[seg];
-    const int col = vt * 64 + j;
+    const int col = vt * C + c;
     const bool live = col < dv;
     const int n_pad = (dk + 3) & ~3;
-    float* st = state + (size_t)row_slot[t0] * state_stride + ((size_t)h * n_tiles + vt) * ((size_t)dk * 64 + n_pad + 4);
-    float* st_n = st + (size_t)dk * 64;
+    float* st = state + (size_t)row_slot[t0] * state_stride + ((size_t)h * n_tiles + vt) * ((size_t)dk * C + n_pad + 4);
+    float* st_n = st + (size_t)dk * C;
     float* st_m = st_n + n_pad;
 
     float S[ROWS], nn[ROWS];
-    const int row0 = r * ROWS;
 #pragma unroll
     for (int rr = 0; rr < ROWS; ++rr) {
-        const int i = row0 + rr;
-        S[rr] = i < dk ? st[(size_t)i * 64 + j] : 0.f;
+        const int i = rr * RG + rg;               // (a lane's rows lie RG apart: the groups' reads of LDS then fall into different banks)
+        S[rr] = i < dk ? st[(size_t)i * C + c] : 0.f;
         nn[rr] = i < dk ? st_n[i] : 0.f;
     }
     float m = st_m[0];
     const float bi = i_bias[h], bf = f_bias[h];
 
-    // the first token's k and q
-    const float* row = proj + (size_t)t0 * ld;
-    if (tid < 4 * ROWS) kq_s[0][tid] = tid < dk ? float2{row[k_off + h * dk + tid], row[q_off + h * dk + tid] * q_scale} : float2{0.f, 0.f};
-    float v_next = live ? row[v_off + h * dv + col] : 0.f;
+    // A block of TB tokens from `first` on (rows beyond the request's last are read as its last: finite, and never used).
+    float2 kq_reg[PER];
+    float v_reg[VPER];
+    auto fetch = [&](int first) {
+#pragma unroll
+        for (int e = 0; e < PER; ++e) {
+            const int idx = lane + 64 * e, u = idx / KQ, i = idx % KQ;
+            const float* row = proj + (size_t)(t0 + min(first + u, n - 1)) * ld;
+            const int ic = min(i, dk - 1);
+            const float kk = row[k_off + h * dk + ic], qq = row[q_off + h * dk + ic] * q_scale;
+            kq_reg[e] = i < dk ? float2{kk, qq} : float2{0.f, 0.f};
+        }
+#pragma unroll
+        for (int e = 0; e < VPER; ++e) {
+            const int idx = min(lane + 64 * e, TB * C - 1), u = idx / C, cc = min(vt * C + idx % C, dv - 1);
+            v_reg[e] = proj[(size_t)(t0 + min(first + u, n - 1)) * ld + v_off + h * dv + cc];
+        }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int e = 0; e < PER; ++e) {
+            const int idx = lane + 64 * e;
+            kq_s[buf][idx / KQ][idx % KQ] = kq_reg[e];
+        }
+#pragma unroll
+        for (int e = 0; e < VPER; ++e) {
+            const int idx = lane + 64 * e;
+            if (idx < TB * C) v_s[buf][idx / C][idx % C] = v_reg[e];
+        }
+    };
+    fetch(0);
+    stash(0);
+    int buf = 0;
 
     for (int b0 = 0; b0 < n; b0 += 64) {
         const int count = min(64, n - b0);
-        if (tid < count) {                           // (wave 0: the gates of this block's tokens)
-            const float* g = proj + (size_t)(t0 + b0 + tid) * ld;
-            gate_i[tid] = cap * tanhf((g[i_off + h] + bi) / cap);
-            gate_f[tid] = log_sigmoid(cap * tanhf((g[f_off + h] + bf) / cap));
-        }
-        __syncthreads();
+        // The gates of this block's tokens, lane u token u; then m along the block, one token after the other (two numbers a
+        // token: cheap), each lane keeping the m before and after its own token; then the exponentials, all tokens at once.
+        const float* g = proj + (size_t)(t0 + b0 + min(lane, count - 1)) * ld;
+        const float li = cap * tanhf((g[i_off + h] + bi) / cap);
+        const float lf = log_sigmoid(cap * tanhf((g[f_off + h] + bf) / cap));
+        float m_before = 0.f, m_after = 0.f;
         for (int u = 0; u < count; ++u) {
-            const int t = t0 + b0 + u, buf = u & 1;
-            const bool more = b0 + u + 1 < n;
-            const float* next = proj + (size_t)(t + (more ? 1 : 0)) * ld;
-            float2 kq_next = {0.f, 0.f};
-            if (tid < dk) kq_next = float2{next[k_off + h * dk + tid], next[q_off + h * dk + tid] * q_scale};
-            const float v_j = v_next;
-            v_next = live ? next[v_off + h * dv + col] : 0.f;
-
-            const float ig = gate_i[u], fg = gate_f[u];
-            const float m_new = fmaxf(fg + m, ig);
-            const float a = expf(fg + m - m_new), b = expf(ig - m_new);
+            const float m_new = fmaxf(lane_value(lf, u) + m, lane_value(li, u));        // (u is the same for the whole wave)
+            if (lane == u) { m_before = m; m_after = m_new; }
             m = m_new;
-            const float bv = b * v_j;
-            float acc = 0.f, nq = 0.f;
+        }
+        __syncthreads();                             // (one wave: orders this block's reads of coef before the writes)
+        coef[lane] = float4{expf(lf + m_before - m_after), expf(li - m_after), expf(-m_after), 0.f};
+        __syncthreads();
+        for (int s0 = 0; s0 < count; s0 += TB, buf ^= 1) {
+            const bool more = b0 + s0 + TB < n;
+            if (more) fetch(b0 + s0 + TB);
+            const int here = min(TB, count - s0);
+            // One token: the memory takes it in; the lane's shares of S^T q and n . q come back, and exp(-m).
+            auto token = [&](int u, float& acc, float& nq, float& floor_) {
+                const float4 cf = coef[s0 + u];
+                const float a = cf.x, b = cf.y;
+                const float bv = b * v_s[buf][u][c];
+                acc = 0.f, nq = 0.f, floor_ = cf.z;
 #pragma unroll
-            for (int rr = 0; rr < ROWS; ++rr) {
-                const float2 kq = kq_s[buf][row0 + rr];
-                S[rr] = fmaf(a, S[rr], kq.x * bv);
-                acc = fmaf(S[rr], kq.y, acc);
-                nn[rr] = fmaf(a, nn[rr], b * kq.x);
-                nq = fmaf(nn[rr], kq.y, nq);
+                for (int rr = 0; rr < ROWS; ++rr) {
+                    const float2 kq = kq_s[buf][u][rr * RG + rg];
+                    S[rr] = fmaf(a, S[rr], kq.x * bv);
+                    acc = fmaf(S[rr], kq.y, acc);
+                    nn[rr] = fmaf(a, nn[rr], b * kq.x);
+                    nq = fmaf(nn[rr], kq.y, nq);
+                }
+            };
+            // UB tokens at a time, so that their reads of LDS go out together.
+            constexpr int UB = TB >= 4 ? 4 : TB;
+            int u = 0;
+            for (; u + UB <= here; u += UB) {
+                float acc[UB], nq[UB], floor_[UB];
+#pragma unroll
+                for (int k = 0; k < UB; ++k) token(u + k, acc[k], nq[k], floor_[k]);
+#pragma unroll
+                for (int k = 0; k < UB; ++k) {
+                    acc[k] = group_sum<RG>(acc[k]);
+                    nq[k] = group_sum<RG>(nq[k]);
+                }
+                if (rg == 0 && live) {
+#pragma unroll
+                    for (int k = 0; k < UB; ++k) out[(size_t)(t0 + b0 + s0 + u + k) * ldo + h * dv + col] = acc[k] / (fmaxf(fabsf(nq[k]), floor_[k]) + 1e-6f);
+                }
             }
-            red[buf][r][j] = acc;
-            if (j == 0) red_n[buf][r] = nq;
-            if (tid < 4 * ROWS) kq_s[buf ^ 1][tid] = kq_next;
+            for (; u < here; ++u) {
+                float acc, nq, floor_;
+                token(u, acc, nq, floor_);
+                acc = group_sum<RG>(acc);
+                nq = group_sum<RG>(nq);
+                if (rg == 0 && live) out[(size_t)(t0 + b0 + s0 + u) * ldo + h * dv + col] = acc / (fmaxf(fabsf(nq), floor_) + 1e-6f);
+            }
+            __syncthreads();                         // this block's reads are done before the buffer after next is written
+            if (more) stash(buf ^ 1);
             __syncthreads();
-            if (r == 0 && live) {
-                const float num = (red[buf][0][j] + red[buf][1][j]) + (red[buf][2][j] + red[buf][3][j]);
-                const float dot = (red_n[buf][0] + red_n[buf][1]) + (red_n[buf][2] + red_n[buf][3]);
-                out[(size_t)t * ldo + h * dv + col] = num / (fmaxf(fabsf(dot), expf(-m)) + 1e-6f);
-            }
         }
     }
 #pragma unroll
     for (int rr = 0; rr < ROWS; ++rr) {
-        const int i = row0 + rr;
+        const int i = rr * RG + rg;               // (a lane's rows lie RG apart: the groups' reads of LDS then fall into different banks)
         if (i < dk) {
-            st[(size_t)i * 64 + j] = S[rr];
-            if (j == 0) st_n[i] = nn[rr];
+            if (live) st[(size_t)i * C + c] = S[rr];
+            if (c == 0) st_n[i] = nn[rr];
         }
     }
-    if (tid == 0) st_m[0] = m;
+    if (lane == 0) st_m[0] = m;
 }
 
 // y[t, h*dv + d] = w[h*dv + d] * o[t, h, d] * rsqrt(mean_d(o[t, h, :]^2) + eps) * sigmoid(g[t, h*dv + d]): one wave per (row, head).
@@ -153,9 +233,13 @@ GI_API int gi_segments(const int* slot, const int* pos, int n_rows, int* seg_sta
     return 0;
 }
 
+// Columns of S a wave owns, by the keys' length.
+static int mlstm_tile(int dk) { return dk <= 32 ? 16 : dk <= 64 ? 8 : 4; }
+
 // Floats of one request slot's state for `n_heads` heads of dk x dv.
 GI_API long gi_mlstm_state_floats(int n_heads, int dk, int dv) {
-    return (long)n_heads * ((dv + 63) / 64) * ((long)dk * 64 + ((dk + 3) & ~3) + 4);
+    const int c = mlstm_tile(dk);
+    return (long)n_heads * ((dv + c - 1) / c) * ((long)dk * c + ((dk + 3) & ~3) + 4);
 }
 
 GI_API int gi_mlstm_max_key_dim() { return 256; }
@@ -167,12 +251,12 @@ GI_API int gi_mlstm_scan(const float* proj, long ld, int q_off, int k_off, int v
                          long state_stride, float* out, long ldo, int n_heads, int dk, int dv, hipStream_t stream) {
     GI_REQUIRE(n_segs > 0 && n_heads > 0 && dk > 0 && dk <= 256 && dv > 0, "mlstm_scan: bad sizes (runs %d, heads %d, dk %d, dv %d; dk at most 256)", n_segs, n_heads, dk, dv);
     GI_REQUIRE(cap > 0.f && state_stride >= gi_mlstm_state_floats(n_heads, dk, dv) && ldo >= (long)n_heads * dv, "mlstm_scan: bad cap, state stride or output stride");
-    const int tiles = (dv + 63) / 64;
+    const int c = mlstm_tile(dk), tiles = (dv + c - 1) / c;
     GI_REQUIRE(n_heads <= 65535 && tiles <= 65535, "mlstm_scan: too many heads or value channels");
     dim3 grid(n_segs, n_heads, tiles);
-#define GO(R) mlstm_scan_kernel<R><<<grid, 256, 0, stream>>>(proj, ld, q_off, k_off, v_off, i_off, f_off, i_bias, f_bias, cap, q_scale, seg_start, seg_len, \
-                                                            row_slot, state, state_stride, out, ldo, dk, dv)
-    if (dk <= 32) GO(8); else if (dk <= 64) GO(16); else if (dk <= 128) GO(32); else GO(64);
+#define GO(C_, R) mlstm_scan_kernel<C_, R><<<grid, 64, 0, stream>>>(proj, ld, q_off, k_off, v_off, i_off, f_off, i_bias, f_bias, cap, q_scale, seg_start, seg_len, \
+                                                                   row_slot, state, state_stride, out, ldo, dk, dv)
+    if (dk <= 32) GO(16, 8); else if (dk <= 64) GO(8, 8); else if (dk <= 128) GO(4, 8); else GO(4, 16);
 #undef GO
     GI_CHECK_LAUNCH("mlstm_scan");
     return 0;

@@ -5,8 +5,8 @@ Matrices are 0.2 * N(0, 1), which makes scores and logits of order one; norm wei
 sinks are of order one so that leaving one out shows.  The configurations differ from one another in every size and option:
 value heads smaller and larger than key heads, one and several key/value heads, rotations of a part of the head and of all of
 it, with and without stretched frequencies, chunks shorter than a page and no multiple of one, layers with and without a
-feed-forward, readers of other layers' keys with the same and with another chunk, memories whose value heads fill a tile of
-64 channels partly, exactly and more than once, key heads that are no multiple of 4."""
+feed-forward, readers of other layers' keys with the same and with another chunk, memories whose value heads are no multiple of
+the kernel's tiles, key heads that are no multiple of 4, and one configuration whose sizes are multiples of nothing."""
 from __future__ import annotations
 
 import json
@@ -54,8 +54,14 @@ FEKORAX_C = dict(architecture="Fekorax", vocab=512, width=128, embedding=dict(sc
     _layer("attention", _attention(4, 2, 64, 64, 0.11, dict(dims=32, base=10000.0), chunk=64, kv_from=0)),
     _layer("attention", _attention(2, 2, 64, 64, 0.125, dict(dims=64, base=500.0), chunk=80), ff=128),
 ])
-CONFIGS = {"A": FEKORAX_A, "B": FEKORAX_B, "C": FEKORAX_C}
-PAGE_SIZE = {"A": 4, "B": 8, "C": 16}
+# Sizes that are multiples of nothing: rows of 50 numbers, heads of 6 and 3 channels, five heads, a chunk of 5 positions.
+FEKORAX_D = dict(architecture="Fekorax", vocab=211, width=50, embedding=dict(scale=1.0), norm=dict(eps=1e-4), layers=[
+    _layer("mlstm", dict(heads=5, dim=3, vdim=5, gate_cap=4.0), ff=30),
+    _layer("attention", _attention(5, 5, 6, 10, 0.5, dict(dims=2, base=7.0, scaling=dict(factor=2.0, low=1.0, high=3.0, original=8)), chunk=5)),
+    _layer("attention", _attention(5, 1, 10, 6, 0.3, dict(dims=6, base=9.0)), ff=22),
+])
+CONFIGS = {"A": FEKORAX_A, "B": FEKORAX_B, "C": FEKORAX_C, "D": FEKORAX_D}
+PAGE_SIZE = {"A": 4, "B": 8, "C": 16, "D": 16}
 
 
 def tensor_layout(cfg):

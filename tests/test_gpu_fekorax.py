@@ -238,11 +238,11 @@ def test_small_kernels():
 
 
 # ================================================================================================= whole models
-LENGTHS = {"A": 90, "B": 75, "C": 150}
+LENGTHS = {"A": 90, "B": 75, "C": 150, "D": 70}
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_prompts_decoding_and_portions_agree_with_the_plain_model(folders, name, dtype):
     cfg = CONFIGS[name]
     tokens = _prompt(cfg, LENGTHS[name], 3)
