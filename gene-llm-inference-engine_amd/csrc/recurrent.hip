@@ -6,14 +6,16 @@
 //     S_t = exp(f_t + m_(t-1) - m_t) S_(t-1) + exp(i_t - m_t) k_t v_t^T        n_t likewise with k_t alone
 //     o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6)
 // with i_t = cap * tanh(pre_i / cap) and f_t = logsigmoid(cap * tanh(pre_f / cap)); S, n and m are zero at a sequence's start
-// (m = 0, not minus infinity).  Columns of S never meet, so one wave owns C of them (a "tile": 16, 8 or 4, fewer for longer
-// keys) for one head of one request and walks the request's rows of this step in order; it keeps its own copy of n and m,
-// which every tile of the head computes alike.  State of one request slot: [head][tile]{S tile [dk][C], n [dk, padded to 4],
-// m, 3 unused}, 32-bit.
+// (m = 0, not minus infinity).  Columns of S never meet, and n is the column that S would have for a value that is always 1.
+// So one wave owns a "tile" of four columns, three of S and n, for one head of one request, and walks the request's rows of this
+// step in order; every tile of a head computes n and m alike and keeps its own copy (a tile that read them from a common place
+// would race with the tile that writes them).  State of one request slot: [head][tile]{[dk][4], m, 3 unused}, 32-bit.
 //
-// Lane = (column, group of rows): a lane keeps ROWS rows (RG apart) of one column in registers, the 64/C groups' shares of S^T q and
-// n . q (neighbouring lanes) are added by the vector unit's lane moves, so a token costs no barrier and no trip through LDS
-// for the sums, and the chip gets heads * dv / C independent waves.
+// Lane = (column, group of rows): a lane keeps ROWS rows (16 apart) of one column in registers; the 16 groups' shares of a
+// column's S^T q (neighbouring lanes) are added by the vector unit's lane moves, and n . q, which every column's output is
+// divided by, is read from the last column's lane.  A token so costs no barrier and no trip through LDS for the sums, three
+// instructions per row of a lane, and the chip gets heads * dv / 3 independent waves: the recurrence is sequential in the
+// tokens, so what counts is how few instructions a wave spends on one.
 // Per token k and q*scale come through LDS (read as broadcasts).  The k, q and v of a block of tokens are asked for while the
 // block before it is worked on and laid into LDS at its end, so that no token waits for memory.  The gates of 64 tokens are made
 // at once, lane by token: m runs along them one after the other (an addition and a maximum each), and the exponentials it needs
@@ -63,18 +65,18 @@ __device__ __forceinline__ float group_sum(float x) {
 
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
-template <int C, int ROWS>
+template <int ROWS>
 __global__ __launch_bounds__(64) void mlstm_scan_kernel(const float* __restrict__ proj, long ld, int q_off, int k_off, int v_off, int i_off, int f_off,
                                                        const float* __restrict__ i_bias, const float* __restrict__ f_bias, float cap, float q_scale,
                                                        const int* __restrict__ seg_start, const int* __restrict__ seg_len,
                                                        const int* __restrict__ row_slot, float* __restrict__ state, long state_stride,
                                                        float* __restrict__ out, long ldo, int dk, int dv) {
+    constexpr int C = 4, VC = 3;                 // columns a wave holds: three of S and n (as the column of a value that is always 1)
     constexpr int RG = 64 / C;                   // groups of rows: lane = column * RG + group, so that a column's groups are neighbouring lanes
     constexpr int KQ = RG * ROWS;                // rows a token's k and q cover (dk, padded with zeros)
     constexpr int TB = 1024 / KQ;                // tokens staged at a time: their k, q and v wait in LDS while the block before them is worked on
     constexpr int PER = TB * KQ / 64;            // (k, q) pairs a lane brings per block
-    static_assert(TB >= 2 && TB <= 64 && 64 % TB == 0, "staging blocks divide the gates' blocks of 64 tokens");
-    constexpr int VPER = (TB * C + 63) / 64;     // values a lane brings per block
+    static_assert(TB >= 2 && TB <= 16 && 64 % TB == 0 && TB * VC <= 64, "staging blocks divide the gates' blocks of 64 tokens; a lane brings one value");
     __shared__ float2 kq_s[2][TB][KQ];
     __shared__ float v_s[2][TB][C];
     __shared__ float4 coef[64];                  // per token of the gates' block: {decay of what is held, weight of what comes, exp(-m), -}
@@ -83,26 +85,23 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(const float* __restrict_
     const int n = seg_len[seg];
     if (n <= 0) return;
     const int t0 = seg_start[seg];
-    const int col = vt * C + c;
-    const bool live = col < dv;
-    const int n_pad = (dk + 3) & ~3;
-    float* st = state + (size_t)row_slot[t0] * state_stride + ((size_t)h * n_tiles + vt) * ((size_t)dk * C + n_pad + 4);
-    float* st_n = st + (size_t)dk * C;
-    float* st_m = st_n + n_pad;
+    const int col = vt * VC + c;
+    const bool live = c < VC && col < dv;
+    float* st = state + (size_t)row_slot[t0] * state_stride + ((size_t)h * n_tiles + vt) * ((size_t)dk * C + 4);
+    float* st_m = st + (size_t)dk * C;
 
-    float S[ROWS], nn[ROWS];
+    float S[ROWS];
 #pragma unroll
     for (int rr = 0; rr < ROWS; ++rr) {
-        const int i = rr * RG + rg;               // (a lane's rows lie RG apart: the groups' reads of LDS then fall into different banks)
+        const int i = rr * RG + rg;                  // (a lane's rows lie RG apart: the groups' reads of LDS then fall into different banks)
         S[rr] = i < dk ? st[(size_t)i * C + c] : 0.f;
-        nn[rr] = i < dk ? st_n[i] : 0.f;
     }
     float m = st_m[0];
     const float bi = i_bias[h], bf = f_bias[h];
 
     // A block of TB tokens from `first` on (rows beyond the request's last are read as its last: finite, and never used).
     float2 kq_reg[PER];
-    float v_reg[VPER];
+    float v_reg;
     auto fetch = [&](int first) {
 #pragma unroll
         for (int e = 0; e < PER; ++e) {
@@ -112,11 +111,8 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(const float* __restrict_
             const float kk = row[k_off + h * dk + ic], qq = row[q_off + h * dk + ic] * q_scale;
             kq_reg[e] = i < dk ? float2{kk, qq} : float2{0.f, 0.f};
         }
-#pragma unroll
-        for (int e = 0; e < VPER; ++e) {
-            const int idx = min(lane + 64 * e, TB * C - 1), u = idx / C, cc = min(vt * C + idx % C, dv - 1);
-            v_reg[e] = proj[(size_t)(t0 + min(first + u, n - 1)) * ld + v_off + h * dv + cc];
-        }
+        const int idx = min(lane, TB * VC - 1), u = idx / VC, cc = min(vt * VC + idx % VC, dv - 1);
+        v_reg = proj[(size_t)(t0 + min(first + u, n - 1)) * ld + v_off + h * dv + cc];
     };
     auto stash = [&](int buf) {
 #pragma unroll
@@ -124,12 +120,9 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(const float* __restrict_
             const int idx = lane + 64 * e;
             kq_s[buf][idx / KQ][idx % KQ] = kq_reg[e];
         }
-#pragma unroll
-        for (int e = 0; e < VPER; ++e) {
-            const int idx = lane + 64 * e;
-            if (idx < TB * C) v_s[buf][idx / C][idx % C] = v_reg[e];
-        }
+        if (lane < TB * VC) v_s[buf][lane / VC][lane % VC] = v_reg;
     };
+    if (lane < 2 * TB) v_s[lane / TB][lane % TB][VC] = 1.0f;          // the value that makes a column of S the normaliser n
     fetch(0);
     stash(0);
     int buf = 0;
@@ -154,44 +147,37 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(const float* __restrict_
             const bool more = b0 + s0 + TB < n;
             if (more) fetch(b0 + s0 + TB);
             const int here = min(TB, count - s0);
-            // One token: the memory takes it in; the lane's shares of S^T q and n . q come back, and exp(-m).
-            auto token = [&](int u, float& acc, float& nq, float& floor_) {
+            // One token: the memory takes it in; the lane's share of its column's S^T q comes back (of n . q in the last column).
+            auto token = [&](int u, float& acc, float& floor_) {
                 const float4 cf = coef[s0 + u];
-                const float a = cf.x, b = cf.y;
-                const float bv = b * v_s[buf][u][c];
-                acc = 0.f, nq = 0.f, floor_ = cf.z;
+                const float a = cf.x, bv = cf.y * v_s[buf][u][c];
+                acc = 0.f, floor_ = cf.z;
 #pragma unroll
                 for (int rr = 0; rr < ROWS; ++rr) {
                     const float2 kq = kq_s[buf][u][rr * RG + rg];
                     S[rr] = fmaf(a, S[rr], kq.x * bv);
                     acc = fmaf(S[rr], kq.y, acc);
-                    nn[rr] = fmaf(a, nn[rr], b * kq.x);
-                    nq = fmaf(nn[rr], kq.y, nq);
                 }
             };
-            // UB tokens at a time, so that their reads of LDS go out together.
-            constexpr int UB = TB >= 4 ? 4 : TB;
+            // The groups' shares are added by lane moves; n . q is then in the last column's lanes, the same for the whole wave.
+            auto finish = [&](int u, float acc, float floor_) {
+                acc = group_sum<RG>(acc);
+                const float x = fmaxf(fabsf(lane_value(acc, VC * RG)), floor_) + 1e-6f;
+                if (rg == 0 && live) out[(size_t)(t0 + b0 + s0 + u) * ldo + h * dv + col] = acc / x;
+            };
+            constexpr int UB = TB >= 4 ? 4 : TB;     // so many tokens at a time, so that their reads of LDS go out together
             int u = 0;
             for (; u + UB <= here; u += UB) {
-                float acc[UB], nq[UB], floor_[UB];
+                float acc[UB], floor_[UB];
 #pragma unroll
-                for (int k = 0; k < UB; ++k) token(u + k, acc[k], nq[k], floor_[k]);
+                for (int k = 0; k < UB; ++k) token(u + k, acc[k], floor_[k]);
 #pragma unroll
-                for (int k = 0; k < UB; ++k) {
-                    acc[k] = group_sum<RG>(acc[k]);
-                    nq[k] = group_sum<RG>(nq[k]);
-                }
-                if (rg == 0 && live) {
-#pragma unroll
-                    for (int k = 0; k < UB; ++k) out[(size_t)(t0 + b0 + s0 + u + k) * ldo + h * dv + col] = acc[k] / (fmaxf(fabsf(nq[k]), floor_[k]) + 1e-6f);
-                }
+                for (int k = 0; k < UB; ++k) finish(u + k, acc[k], floor_[k]);
             }
             for (; u < here; ++u) {
-                float acc, nq, floor_;
-                token(u, acc, nq, floor_);
-                acc = group_sum<RG>(acc);
-                nq = group_sum<RG>(nq);
-                if (rg == 0 && live) out[(size_t)(t0 + b0 + s0 + u) * ldo + h * dv + col] = acc / (fmaxf(fabsf(nq), floor_) + 1e-6f);
+                float acc, floor_;
+                token(u, acc, floor_);
+                finish(u, acc, floor_);
             }
             __syncthreads();                         // this block's reads are done before the buffer after next is written
             if (more) stash(buf ^ 1);
@@ -200,11 +186,8 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(const float* __restrict_
     }
 #pragma unroll
     for (int rr = 0; rr < ROWS; ++rr) {
-        const int i = rr * RG + rg;               // (a lane's rows lie RG apart: the groups' reads of LDS then fall into different banks)
-        if (i < dk) {
-            if (live) st[(size_t)i * C + c] = S[rr];
-            if (c == 0) st_n[i] = nn[rr];
-        }
+        const int i = rr * RG + rg;
+        if (i < dk && (live || c == VC)) st[(size_t)i * C + c] = S[rr];
     }
     if (lane == 0) st_m[0] = m;
 }
@@ -233,30 +216,26 @@ GI_API int gi_segments(const int* slot, const int* pos, int n_rows, int* seg_sta
     return 0;
 }
 
-// Columns of S a wave owns, by the keys' length.
-static int mlstm_tile(int dk) { return dk <= 32 ? 16 : dk <= 64 ? 8 : 4; }
-
-// Floats of one request slot's state for `n_heads` heads of dk x dv.
+// Floats of one request slot's state for `n_heads` heads of dk x dv: per head and tile of three value channels, [dk][4] and m (padded to 4).
 GI_API long gi_mlstm_state_floats(int n_heads, int dk, int dv) {
-    const int c = mlstm_tile(dk);
-    return (long)n_heads * ((dv + c - 1) / c) * ((long)dk * c + ((dk + 3) & ~3) + 4);
+    return (long)n_heads * ((dv + 2) / 3) * ((long)dk * 4 + 4);
 }
 
-GI_API int gi_mlstm_max_key_dim() { return 256; }
+GI_API int gi_mlstm_max_key_dim() { return 512; }
 
 // proj: float32 [n_rows, ld], whose columns q_off.. hold q [heads*dk], k_off.. k [heads*dk], v_off.. v [heads*dv], i_off.. and
 // f_off.. the gates' pre-activations [heads]; out: float32 [n_rows, ldo] gets o [heads*dv]; state: [slots, state_stride].
 GI_API int gi_mlstm_scan(const float* proj, long ld, int q_off, int k_off, int v_off, int i_off, int f_off, const float* i_bias, const float* f_bias,
                          float cap, float q_scale, const int* seg_start, const int* seg_len, int n_segs, const int* row_slot, float* state,
                          long state_stride, float* out, long ldo, int n_heads, int dk, int dv, hipStream_t stream) {
-    GI_REQUIRE(n_segs > 0 && n_heads > 0 && dk > 0 && dk <= 256 && dv > 0, "mlstm_scan: bad sizes (runs %d, heads %d, dk %d, dv %d; dk at most 256)", n_segs, n_heads, dk, dv);
+    GI_REQUIRE(n_segs > 0 && n_heads > 0 && dk > 0 && dk <= 512 && dv > 0, "mlstm_scan: bad sizes (runs %d, heads %d, dk %d, dv %d; dk at most 512)", n_segs, n_heads, dk, dv);
     GI_REQUIRE(cap > 0.f && state_stride >= gi_mlstm_state_floats(n_heads, dk, dv) && ldo >= (long)n_heads * dv, "mlstm_scan: bad cap, state stride or output stride");
-    const int c = mlstm_tile(dk), tiles = (dv + c - 1) / c;
+    const int tiles = (dv + 2) / 3;
     GI_REQUIRE(n_heads <= 65535 && tiles <= 65535, "mlstm_scan: too many heads or value channels");
     dim3 grid(n_segs, n_heads, tiles);
-#define GO(C_, R) mlstm_scan_kernel<C_, R><<<grid, 64, 0, stream>>>(proj, ld, q_off, k_off, v_off, i_off, f_off, i_bias, f_bias, cap, q_scale, seg_start, seg_len, \
-                                                                   row_slot, state, state_stride, out, ldo, dk, dv)
-    if (dk <= 32) GO(16, 8); else if (dk <= 64) GO(8, 8); else if (dk <= 128) GO(4, 8); else GO(4, 16);
+#define GO(R) mlstm_scan_kernel<R><<<grid, 64, 0, stream>>>(proj, ld, q_off, k_off, v_off, i_off, f_off, i_bias, f_bias, cap, q_scale, seg_start, seg_len, \
+                                                           row_slot, state, state_stride, out, ldo, dk, dv)
+    if (dk <= 64) GO(4); else if (dk <= 128) GO(8); else if (dk <= 256) GO(16); else GO(32);
 #undef GO
     GI_CHECK_LAUNCH("mlstm_scan");
     return 0;

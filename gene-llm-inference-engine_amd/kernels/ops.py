@@ -524,14 +524,13 @@ def segments(ctx):
 
 
 def mlstm_state_floats(n_heads, dk, dv) -> int:
-    """32-bit numbers of one request's matrix memories, as `mlstm_scan` lays them out for itself: per head and tile of C value
-    channels (C = 16, 8 or 4: fewer for longer keys) the tile of S, n padded to a multiple of 4, m and 3 unused (the library's
-    `gi_mlstm_state_floats` says the same; this one needs no library, so that a cache can be planned without one)."""
-    c = 16 if dk <= 32 else 8 if dk <= 64 else 4
-    return n_heads * (-(-dv // c)) * (dk * c + ((dk + 3) & ~3) + 4)
+    """32-bit numbers of one request's matrix memories, as `mlstm_scan` lays them out for itself: per head and tile of three value
+    channels, [dk][4] (three columns of S and the normaliser n) and m padded to four numbers (the library's `gi_mlstm_state_floats`
+    says the same; this one needs no library, so that a cache can be planned without one)."""
+    return n_heads * (-(-dv // 3)) * (dk * 4 + 4)
 
 
-MLSTM_MAX_KEY_DIM = 256
+MLSTM_MAX_KEY_DIM = 512
 
 
 def mlstm_max_key_dim() -> int:

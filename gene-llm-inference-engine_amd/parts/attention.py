@@ -132,9 +132,10 @@ class Attention(Mixer):
     @classmethod
     def tensor_needs(cls, spec):
         a, kv, d, vd = spec.n_heads * spec.head_dim, spec.n_kv_heads * spec.head_dim, spec.hidden_size, spec.value_dim or spec.head_dim
-        needs = [TensorNeed(spec.q_proj, (a, d)), TensorNeed(spec.o_proj, (d, spec.n_heads * vd))]
+        needs = [TensorNeed(spec.q_proj, (a, d))]
         if spec.k_proj is not None:            # (a layer that reads another layer's pages has no keys and values of its own)
             needs += [TensorNeed(spec.k_proj, (kv, d)), TensorNeed(spec.v_proj, (spec.n_kv_heads * vd, d))]
+        needs.append(TensorNeed(spec.o_proj, (d, spec.n_heads * vd)))
         if spec.q_norm is not None:
             needs.append(TensorNeed(spec.q_norm, (spec.head_dim,), "norm"))
         if spec.k_norm is not None and spec.k_proj is not None:

@@ -369,3 +369,63 @@ def test_matrix_core_attention_with_chunks_sinks_and_gates(hd, heads, kv, chunk)
         assert relative_error(fast.float(), slow.float()) < 2e-2, sorted(extras)
         worst = (fast.float() - slow.float()).abs().view(T, heads, hd).amax(dim=(1, 2))
         assert float(worst.max()) < 0.06, (sorted(extras), int(worst.argmax()))
+
+
+@pytest.mark.parametrize("dtype, mode", [("float32", "mixed"), ("bfloat16", "mixed"), ("float32", "portions")])
+def test_replay_through_the_command_line(folders, tmp_path, dtype, mode):
+    """bin/trace_run as a child process on a Fekorax folder: up to four live requests, portions beside single tokens, a pool that
+    holds less than all requests together, so that pages and state slots are used again."""
+    import json
+    import random
+    import subprocess
+    from pathlib import Path
+    import numpy as np
+    import traces
+    root = Path(__file__).resolve().parent.parent
+    cfg = CONFIGS["A"]
+    rng = random.Random(4)
+    requests = {f"q{i}": [rng.randrange(cfg["vocab"]) for _ in range(n)] for i, n in enumerate([50, 1, 33, 77, 40, 9])}
+    steps = traces.mixed(requests, seed=3) if mode == "mixed" else traces.portions(requests)
+    out = tmp_path / "out"
+    cmd = [str(root / "bin" / "trace_run"), "--model", str(folders["A"]), "--dtype", dtype, "--out", str(out), "--max-tokens", str(traces.peak_tokens(steps, 64)),
+           "--page-size", "4"]
+    proc = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+    try:
+        for s in steps:
+            proc.stdin.write(json.dumps(s) + "\n")
+            proc.stdin.flush()
+            line = proc.stdout.readline().strip()
+            assert line == f"done {s['step']}", (line, proc.stderr.read() if proc.poll() is not None else "")
+        proc.stdin.close()
+        assert proc.wait(timeout=60) == 0, proc.stderr.read()
+    finally:
+        if proc.poll() is None:
+            proc.kill()
+    got = {}
+    for step, rows in traces.wanted_positions(steps).items():
+        data = np.fromfile(out / f"{step}.f32", dtype="<f4").reshape(len(rows), cfg["vocab"])
+        for key, row in zip(rows, data):
+            got[key] = torch.from_numpy(row.copy())
+    for rid, tokens in requests.items():
+        mine = {p: row for (r, p), row in got.items() if r == rid}
+        assert len(mine) > 0
+        exact = plain_logits(folders, "A", tokens)
+        if dtype == "float32":            # (the same bound as `check_against_plain`: four times what the plain model loses in 32-bit)
+            single = plain_logits(folders, "A", tokens, dtype=torch.float32)
+            noise = max(relative_error(single[p], exact[p]) for p in mine)
+            assert max(relative_error(row, exact[p]) for p, row in mine.items()) < 4 * noise + 1e-5
+        else:
+            rounded = plain_logits(folders, "A", tokens, rounded=True)
+            assert_within_bfloat16_noise(mine, lambda p: exact[p], lambda p: rounded[p], f"replay {mode} {rid}")
+
+
+def test_generation_from_the_command_line_on_random_weights(tmp_path):
+    """bin/gi_generate on the shipped example configuration, random weights, greedy: runs, and twice the same."""
+    import subprocess
+    from pathlib import Path
+    root = Path(__file__).resolve().parent.parent
+    cmd = [str(root / "bin" / "gi_generate"), "--config", str(root / "configs" / "fekorax-small.json"), "--random-seed", "3", "--prompt-ids", "5 17 3 999 4",
+           "--steps", "24", "--temperature", "0"]
+    runs = [subprocess.run(cmd, capture_output=True, text=True, timeout=280) for _ in range(2)]
+    assert all(r.returncode == 0 for r in runs), runs[0].stderr[-2000:]
+    assert runs[0].stdout == runs[1].stdout and len(runs[0].stdout.split()) >= 20
