@@ -64,7 +64,7 @@ def fekorax_beside_llama(args) -> int:
         att = lambda source=None: dict(type="attention", mlp=dict(kind="dense", ff=ff), mixer=dict(
             heads=H, kv_heads=G, dim=hd, vdim=hd, scale=hd ** -0.5, rot=dict(dims=hd // 2, base=10000.0), mask=dict(size=1024),
             **({} if source is None else dict(kv_from=source))))
-        mem = dict(type="mlstm", mlp=None, mixer=dict(heads=max(1, H // 4), dim=hd, vdim=2 * hd, gate_cap=15.0))
+        mem = dict(type="mlstm", mlp=None, mixer=dict(heads=max(1, H // 4), dim=hd, vdim=2 * hd, gate_cap=12.0))
         layers = []
         for i in range(0, L, 4):
             layers += [mem, att(), mem, att(i + 1)]

@@ -41,7 +41,7 @@ FEKORAX_A = dict(architecture="Fekorax", vocab=320, width=64, embedding=dict(sca
     _layer("mlstm", dict(heads=4, dim=16, vdim=16, gate_cap=6.0)),
 ])
 FEKORAX_B = dict(architecture="Fekorax", vocab=257, width=96, embedding=dict(scale=0.7), norm=dict(eps=1e-6), layers=[
-    _layer("mlstm", dict(heads=3, dim=20, vdim=72, gate_cap=15.0)),
+    _layer("mlstm", dict(heads=3, dim=20, vdim=72, gate_cap=14.0)),
     _layer("attention", _attention(3, 3, 16, 48, 0.3, dict(dims=16, base=50.0), chunk=7), ff=64),
     _layer("attention", _attention(6, 3, 16, 48, 0.25, dict(dims=16, base=50.0), chunk=13, kv_from=1), ff=48),
     _layer("attention", _attention(2, 1, 24, 24, 0.4)),
