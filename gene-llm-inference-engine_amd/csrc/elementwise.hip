@@ -511,3 +511,44 @@ GI_API int gi_act_mul(const float* gate_up, void* h, int h_dtype, int n_rows, in
     GI_CHECK_LAUNCH("act_mul");
     return 0;
 }
+
+// The same, and on the way the norm that reads the rows next: x += w * norm(y), then out = w_next * norm(x), with out stored as
+// the next product reads it.  A thread reads back only what it wrote itself.
+template <typename TW, typename TO>
+__global__ __launch_bounds__(256) void rmsnorm_add_norm_kernel(const float* __restrict__ y, const TW* __restrict__ w, float* __restrict__ x,
+                                                              const TW* __restrict__ w_next, TO* __restrict__ out, int dim, float eps, float eps_next,
+                                                              size_t y_stride, size_t x_stride, size_t out_stride) {
+    __shared__ float red[4];
+    const float* yr = y + (size_t)blockIdx.x * y_stride;
+    float* xr = x + (size_t)blockIdx.x * x_stride;
+    TO* orow = out + (size_t)blockIdx.x * out_stride;
+    float ss = 0.f;
+    for (int d = threadIdx.x; d < dim; d += 256) ss = fmaf(yr[d], yr[d], ss);
+    ss = block_sum<256>(ss, red);
+    const float scale = 1.0f / sqrtf(ss / (float)dim + eps);
+    float sx = 0.f;
+    for (int d = threadIdx.x; d < dim; d += 256) {
+        const float v = xr[d] + load_f32(w, d) * (scale * yr[d]);
+        xr[d] = v;
+        sx = fmaf(v, v, sx);
+    }
+    sx = block_sum<256>(sx, red);
+    const float scale_next = 1.0f / sqrtf(sx / (float)dim + eps_next);
+    for (int d = threadIdx.x; d < dim; d += 256) store_f32(orow, d, load_f32(w_next, d) * (scale_next * xr[d]));
+}
+
+GI_API int gi_rmsnorm_add_norm(const float* y, const void* w, const void* w_next, int w_dtype, float* x, void* out, int out_dtype, int n_rows, int dim,
+                               float eps, float eps_next, long y_stride, long x_stride, long out_stride, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && dim > 0 && y_stride >= dim && x_stride >= dim && out_stride >= dim, "rmsnorm_add_norm: bad sizes (rows %d, dim %d)", n_rows, dim);
+#define LAUNCH(TW, TO)                                                                                                                            \
+    rmsnorm_add_norm_kernel<TW, TO><<<n_rows, 256, 0, stream>>>(y, (const TW*)w, x, (const TW*)w_next, (TO*)out, dim, eps, eps_next, (size_t)y_stride, \
+                                                                (size_t)x_stride, (size_t)out_stride)
+    if (w_dtype == GI_F32 && out_dtype == GI_F32) LAUNCH(float, float);
+    else if (w_dtype == GI_F32 && out_dtype == GI_BF16) LAUNCH(float, bf16_t);
+    else if (w_dtype == GI_BF16 && out_dtype == GI_F32) LAUNCH(bf16_t, float);
+    else if (w_dtype == GI_BF16 && out_dtype == GI_BF16) LAUNCH(bf16_t, bf16_t);
+    else return gi_fail("rmsnorm_add_norm: unknown dtypes %d, %d", w_dtype, out_dtype);
+#undef LAUNCH
+    GI_CHECK_LAUNCH("rmsnorm_add_norm");
+    return 0;
+}

@@ -37,6 +37,7 @@ _SIGNATURES = {
     "gi_attention_exact": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int,
                            c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_long, c_void_p],
     "gi_rmsnorm_add": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_long, c_long, c_void_p],
+    "gi_rmsnorm_add_norm": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_long, c_long, c_long, c_void_p],
     "gi_norm_rope_store": [c_void_p, c_void_p, c_void_p, c_long, c_long, c_long, c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int,
                            c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gi_act_mul": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
@@ -457,6 +458,20 @@ def rmsnorm_add(y, weight, eps, x):
         raise KernelError("rmsnorm_add: weight must be [dim]")
     _call("gi_rmsnorm_add", y.data_ptr(), weight.data_ptr(), _code(weight, "rmsnorm_add: weight"), x.data_ptr(), n, dim, float(eps), y.stride(0), x.stride(0), _stream())
     return x
+
+
+def rmsnorm_add_norm(y, weight, eps, x, next_weight, next_eps, out):
+    """x += weight * norm(y), and out = next_weight * norm(x) of the rows so made (the norm that reads x next), in one kernel;
+    x and y float32 [n, dim], out [n, dim] float32 or bfloat16, the two weights of one dtype."""
+    _dev(y, weight, x, next_weight, out)
+    n, dim = x.shape
+    if not (x.dtype == torch.float32 and y.dtype == torch.float32 and y.shape == (n, dim) and out.shape == (n, dim) and x.stride(1) == 1 and y.stride(1) == 1 and out.stride(1) == 1):
+        raise KernelError("rmsnorm_add_norm: x and y must be float32 [n, dim] and out [n, dim], with unit inner stride")
+    if not (weight.shape == (dim,) and weight.is_contiguous() and next_weight.shape == (dim,) and next_weight.is_contiguous() and weight.dtype == next_weight.dtype):
+        raise KernelError("rmsnorm_add_norm: the weights must be [dim], of one dtype")
+    _call("gi_rmsnorm_add_norm", y.data_ptr(), weight.data_ptr(), next_weight.data_ptr(), _code(weight, "rmsnorm_add_norm: weight"), x.data_ptr(), out.data_ptr(),
+          _code(out, "rmsnorm_add_norm: out"), n, dim, float(eps), float(next_eps), y.stride(0), x.stride(0), out.stride(0), _stream())
+    return out
 
 
 def norm_rope_store(q, k, v, q_norm, k_norm, eps, cos, sin, rotary_dim, positions, slots, table, q_out, cache, page_size, n_heads, n_kv, hd, vd):

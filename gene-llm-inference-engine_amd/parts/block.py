@@ -11,7 +11,7 @@ import torch
 
 from ..kernels import ops
 from .base import feed_forward_class, mixer_class, norm_class, register_block
-from .norm import norm_to_hand_on
+from .norm import NormedRows, norm_to_hand_on
 
 
 class PreNormBlock:
@@ -117,28 +117,51 @@ class SandwichBlock:
     def cache_need(cls, spec):
         return mixer_class(spec.mixer).cache_need(spec.mixer)
 
+    # The norm behind a half and the norm that reads the rows next (this layer's second, or the next layer's first, or the
+    # model's last when every row's logits are wanted) run as one kernel where both are RMS norms with weights of one dtype:
+    # the block plays the model's game of handing a norm on (`hands_norm_on`, `first_reader`, `handed`, `next_reader`).
+    hands_norm_on = True
+
+    def first_reader(self):
+        return self.mixer_norm, self.mixer
+
     @staticmethod
-    def _half(norm, part, post, x, ctx, *cache):
-        h = PreNormBlock._normed(norm, part, x, ctx)
+    def _half(h, part, post, x, ctx, reader, *cache):
+        """x += post(part(h)); returns the rows `reader` = (norm, part) will read, if they were made on the way, else None."""
+        if isinstance(h, NormedRows) and not getattr(part, "accepts_deferred_norm", False):
+            h = h.materialize()
         if getattr(part, "can_overwrite", False):
             y = torch.empty_like(x)
             part.forward(h, y, ctx, *cache, overwrite=True)
         else:
             y = torch.zeros_like(x)
             part.forward(h, y, ctx, *cache)
+        then, reads = reader if reader is not None else (None, None)
+        if (then is not None and hasattr(post, "add_onto_then") and type(then) is type(post) and then.weight.dtype == post.weight.dtype
+                and then.weight.shape == post.weight.shape):
+            return post.add_onto_then(y, x, then, getattr(reads, "in_dtype", ctx.dtype))
         if hasattr(post, "add_onto"):
             post.add_onto(y, x)
         else:
             x += post(y, torch.float32)
+        return None
 
-    def forward(self, x, ctx, cache):
-        self._half(self.mixer_norm, self.mixer, self.mixer_post_norm, x, ctx, cache)
+    def forward(self, x, ctx, cache, handed=None, next_reader=None):
+        """handed: this block's first norm as whoever wrote x last left it (rows ready to read), or None.  next_reader:
+        `first_reader()` of whatever reads x after this block, or None.  Returns that reader's rows, or None."""
+        if handed is None or handed.norm is not self.mixer_norm:
+            handed = PreNormBlock._normed(self.mixer_norm, self.mixer, x, ctx)
+        inner = (self.feed_forward_norm, self.feed_forward) if self.feed_forward is not None else next_reader
+        handed = self._half(handed, self.mixer, self.mixer_post_norm, x, ctx, inner, cache)
         if ctx.trace is not None:
             ctx.trace("attn_out", x)
         if self.feed_forward is not None:
-            self._half(self.feed_forward_norm, self.feed_forward, self.feed_forward_post_norm, x, ctx)
+            if handed is None:
+                handed = PreNormBlock._normed(self.feed_forward_norm, self.feed_forward, x, ctx)
+            handed = self._half(handed, self.feed_forward, self.feed_forward_post_norm, x, ctx, next_reader)
         if ctx.trace is not None:
             ctx.trace("ffn_out", x)
+        return handed
 
 
 register_block("sandwich", SandwichBlock)

@@ -42,6 +42,14 @@ class HandedRows(NormedRows):
         self.scaled, self.squares, self.eps = scaled, squares, norm.eps
 
 
+class ReadyRows(NormedRows):
+    """norm(x) already computed by whoever wrote x last (a kernel that adds onto x and norms the result in one go)."""
+
+    def __init__(self, norm, x: torch.Tensor, value: torch.Tensor):
+        super().__init__(norm, x, value.dtype)
+        self._value = value
+
+
 def norm_to_hand_on(reader, n_rows: int):
     """reader: (norm, part) as a block's `first_reader()` gives it, or None.  The norm, if whoever writes the rows it reads
     next can apply it half way (`HandedRows`): it has weights to apply so (`handed_weight`) and the part's first product
@@ -79,6 +87,12 @@ class RmsNorm(Norm):
     def add_onto(self, y, x):
         """x += norm(y), both float32 [T, size]: what a layer does whose norm follows a sublayer."""
         return ops.rmsnorm_add(y, self.weight, self.eps, x)
+
+    def add_onto_then(self, y, x, then: "RmsNorm", out_dtype) -> ReadyRows:
+        """x += norm(y), and the rows `then` will read, then(x), made on the way."""
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        ops.rmsnorm_add_norm(y, self.weight, self.eps, x, then.weight, then.eps, out)
+        return ReadyRows(then, x, out)
 
     def deferred(self, x, out_dtype, rows=None) -> NormedRows:
         return NormedRows(self, x, out_dtype, rows)
