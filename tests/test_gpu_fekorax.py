@@ -94,7 +94,7 @@ def test_segments_are_found_on_the_device():
     assert length.tolist() == lens and start.tolist() == [0, 3, 4, 74, 75, 76]
 
 
-@pytest.mark.parametrize("heads, dk, dv", [(2, 20, 72), (3, 64, 64), (1, 130, 40), (2, 7, 200)])
+@pytest.mark.parametrize("heads, dk, dv", [(2, 20, 72), (3, 64, 64), (1, 130, 40), (2, 7, 200), (1, 100, 50), (1, 300, 10)])
 def test_matrix_memory_kernel(heads, dk, dv):
     """Two requests of unequal length in one step; then the longer one again in three steps from a fresh slot: the state carries."""
     from geneinfer_amd.kernels import ops
@@ -227,6 +227,12 @@ def test_small_kernels():
     x, y, w = torch.randn(5, 70, generator=g), torch.randn(5, 70, generator=g), 1 + 0.1 * torch.randn(70, generator=g)
     got = ops.rmsnorm_add(y.to(DEV), w.to(DEV), 1e-5, x.clone().to(DEV)).cpu()
     assert relative_error(got, x.double() + unit_rms(y.double(), 1e-5) * w.double()) < 1e-6
+    w2 = 1 + 0.1 * torch.randn(70, generator=g)
+    for out_dtype, tol in ((torch.float32, 1e-6), (torch.bfloat16, 5e-3)):
+        xs = x.clone().to(DEV)
+        nxt = ops.rmsnorm_add_norm(y.to(DEV), w.to(DEV), 1e-5, xs, w2.to(DEV), 1e-4, torch.empty(5, 70, dtype=out_dtype, device=DEV)).float().cpu()
+        summed = x.double() + unit_rms(y.double(), 1e-5) * w.double()
+        assert relative_error(xs.cpu(), summed) < 1e-6 and relative_error(nxt, unit_rms(summed, 1e-4) * w2.double()) < tol
     gu = 3 * torch.randn(7, 2 * 33, generator=g)
     for name, act in (("gelu_tanh", gelu_tanh), ("silu", torch.nn.functional.silu)):
         out = ops.act_mul(gu.to(DEV), torch.empty(7, 33, device=DEV), name).cpu()
