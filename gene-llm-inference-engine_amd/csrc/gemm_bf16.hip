@@ -34,7 +34,9 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-enum Epilogue : int { EPI_STORE_F32 = 0, EPI_ADD_F32 = 1, EPI_STORE_BF16 = 2, EPI_GATED_BF16 = 3, EPI_QKV_ROPE = 4 };
+enum Epilogue : int { EPI_STORE_F32 = 0, EPI_ADD_F32 = 1, EPI_STORE_BF16 = 2, EPI_GATED_BF16 = 3, EPI_QKV_ROPE = 4, EPI_GATED_GELU_BF16 = 5 };
+// The two gated epilogues differ in the activation alone: SiLU (EPI_GATED_BF16), or the tanh form of GELU.
+__host__ __device__ constexpr bool is_gated(int epi) { return epi == EPI_GATED_BF16 || epi == EPI_GATED_GELU_BF16; }
 
 __device__ __forceinline__ float silu_gate(float g, float u) { return (g * (1.0f / (1.0f + expf(-g)))) * u; }
 // The same with the hardware's exp2 and reciprocal (each within a unit or two in the last place of 32 bits): for results
@@ -43,6 +45,17 @@ __device__ __forceinline__ float silu_gate(float g, float u) { return (g * (1.0f
 __device__ __forceinline__ float silu_gate_fast(float g, float u) {
     return (g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.4426950408889634f))) * u;
 }
+
+// gelu_tanh(g) = 0.5 g (1 + tanh(c (g + 0.044715 g^3))), c = sqrt(2 / pi); 0.5 (1 + tanh z) = 1 / (1 + e^(-2z)) for the quick form.
+__device__ __forceinline__ float gelu_gate(float g, float u) { return (0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)))) * u; }
+__device__ __forceinline__ float gelu_gate_fast(float g, float u) {
+    const float z = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+    return (g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(z * -2.8853900817779268f))) * u;
+}
+template <int EPI>
+__device__ __forceinline__ float gate_of(float g, float u) { return EPI == EPI_GATED_GELU_BF16 ? gelu_gate(g, u) : silu_gate(g, u); }
+template <int EPI>
+__device__ __forceinline__ float gate_fast_of(float g, float u) { return EPI == EPI_GATED_GELU_BF16 ? gelu_gate_fast(g, u) : silu_gate_fast(g, u); }
 
 __device__ __forceinline__ uint4 load16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
 __device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
@@ -304,11 +317,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(const bf16_t* __re
             for (int v = 0; v < 16; ++v) {
                 const int m = m0 + wm + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v & 3);
                 const int n = n0 + wn + j * 32 + (lane & 31);
-                if constexpr (EPI == EPI_GATED_BF16) {
+                if constexpr (is_gated(EPI)) {
                     // columns 32b .. 32b+15 are gates, 32b+16 .. 32b+31 the ups of outputs 16b .. 16b+15
                     const float up = __shfl_xor(acc[i][j][v], 16, 64);
                     if ((lane & 16) == 0 && m < M && n < N)
-                        ((bf16_t*)C)[(size_t)m * ldc + (n >> 5) * 16 + (lane & 15)] = f32_to_bf16(silu_gate(acc[i][j][v], up));
+                        ((bf16_t*)C)[(size_t)m * ldc + (n >> 5) * 16 + (lane & 15)] = f32_to_bf16(gate_of<EPI>(acc[i][j][v], up));
                 } else {
                     if (m < M && n < N) write_out<EPI>(C, (size_t)m * ldc + n, acc[i][j][v]);
                 }
@@ -484,10 +497,10 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_piped_kernel
             for (int v = 0; v < 16; ++v) {
                 const int m = m0 + wm + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v & 3);
                 const int n = n0 + wn + j * 32 + (lane & 31);
-                if constexpr (EPI == EPI_GATED_BF16) {
+                if constexpr (is_gated(EPI)) {
                     const float up = __shfl_xor(acc[i][j][v], 16, 64);
                     if ((lane & 16) == 0 && m < M && n < N)
-                        ((bf16_t*)C)[(size_t)m * ldc + (n >> 5) * 16 + (lane & 15)] = f32_to_bf16(silu_gate(acc[i][j][v], up));
+                        ((bf16_t*)C)[(size_t)m * ldc + (n >> 5) * 16 + (lane & 15)] = f32_to_bf16(gate_of<EPI>(acc[i][j][v], up));
                 } else if constexpr (EPI != EPI_QKV_ROPE) {
                     if (m < M && n < N) write_out<EPI>(C, (size_t)m * ldc + n, acc[i][j][v]);
                 }
@@ -583,8 +596,8 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const bf16_t* _
     // the tile's 256 rows' factors are worked out once, a thread a row (16-byte reads of the row's pieces where they allow it: a lane
     // that asked for its rows' pieces one by one cost the kernel 18 us at 16 pieces), and wait in LDS for the epilogue (asked for behind the first block's loads; the
     // barriers of the loop lie between this write and the epilogue's reads).
-    __shared__ float row_scale[EPI == EPI_GATED_BF16 ? BM : 1];
-    if constexpr (EPI == EPI_GATED_BF16) {
+    __shared__ float row_scale[is_gated(EPI) ? BM : 1];
+    if constexpr (is_gated(EPI)) {
         if (norm_in.squares != nullptr) {
             if (tid < BM) {
                 const float* pieces = norm_in.squares + (size_t)min(m0 + tid, M - 1) * norm_in.parts;
@@ -654,7 +667,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const bf16_t* _
     constexpr int STAGE_ROW = 144;
     unsigned char* mine = ring + wave * (WM * STAGE_ROW);
     const int frow = lane >> 3, fchunk = lane & 7;                                 // the flush: lane -> (row within 8, 16-byte piece of 128)
-    if constexpr (EPI == EPI_GATED_BF16) {
+    if constexpr (is_gated(EPI)) {
         // columns 32b .. 32b+15 are gates, 32b+16 .. 32b+31 the ups of outputs 16b .. 16b+15: element v beside element v + 8.
         // The wave's WN columns become WN/2 outputs: 2 * WN/2 bytes a row, flushed 64 outputs (128 bytes) at a time.
         static_assert(WN % 128 == 0, "the gated flush takes 64 outputs at a time");
@@ -668,8 +681,8 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const bf16_t* _
 #pragma unroll
                     for (int q = 0; q < 2; ++q) {
                         const float rs = norm_in.squares != nullptr ? row_scale[wm + i * 32 + (lane & 31)] : 1.0f;
-                        const uint2 packed = {f32x2_to_bf16x2(silu_gate_fast(acc[i][j][4 * q] * rs, acc[i][j][4 * q + 8] * rs), silu_gate_fast(acc[i][j][4 * q + 1] * rs, acc[i][j][4 * q + 9] * rs)),
-                                              f32x2_to_bf16x2(silu_gate_fast(acc[i][j][4 * q + 2] * rs, acc[i][j][4 * q + 10] * rs), silu_gate_fast(acc[i][j][4 * q + 3] * rs, acc[i][j][4 * q + 11] * rs))};
+                        const uint2 packed = {f32x2_to_bf16x2(gate_fast_of<EPI>(acc[i][j][4 * q] * rs, acc[i][j][4 * q + 8] * rs), gate_fast_of<EPI>(acc[i][j][4 * q + 1] * rs, acc[i][j][4 * q + 9] * rs)),
+                                              f32x2_to_bf16x2(gate_fast_of<EPI>(acc[i][j][4 * q + 2] * rs, acc[i][j][4 * q + 10] * rs), gate_fast_of<EPI>(acc[i][j][4 * q + 3] * rs, acc[i][j][4 * q + 11] * rs))};
                         *reinterpret_cast<uint2*>(mine + (i * 32 + (lane & 31)) * STAGE_ROW + (jj * 16 + 8 * q + 4 * (lane >> 5)) * 2) = packed;
                     }
                 }
@@ -902,7 +915,7 @@ __global__ __launch_bounds__(512, MT == 2 ? 4 : 2) void gemm_bf16_skinny_kernel(
             for (int v = 0; v < 4; ++v) acc[t][v] += other[strip][t][lane][v];
     }
     // Element v of a lane's 16x16 result: row (activation row) 4*(lane/16) + v, column (weight row) lane%16.
-    if constexpr (EPI == EPI_GATED_BF16 && !PARTIAL) {
+    if constexpr (is_gated(EPI) && !PARTIAL) {
         // strips 0 and 2 hold gates, strips 1 and 3 the ups of the same outputs: the ups cross over through LDS
         __syncthreads();
         if (half == 0 && (strip & 1)) {
@@ -919,7 +932,7 @@ __global__ __launch_bounds__(512, MT == 2 ? 4 : 2) void gemm_bf16_skinny_kernel(
                 for (int v = 0; v < 4; ++v) {
                     const int m = t * 16 + 4 * q + v;
                     const float rs = scaled_rows ? row_scale[m] : 1.0f;
-                    if (m < M) ((bf16_t*)C)[(size_t)m * ldc + blockIdx.x * 32 + (strip >> 1) * 16 + r] = f32_to_bf16(silu_gate(acc[t][v] * rs, other[strip + 1][t][lane][v] * rs));
+                    if (m < M) ((bf16_t*)C)[(size_t)m * ldc + blockIdx.x * 32 + (strip >> 1) * 16 + r] = f32_to_bf16(gate_of<EPI>(acc[t][v] * rs, other[strip + 1][t][lane][v] * rs));
                 }
         }
     } else if (half == 0 && n < N) {
@@ -1020,7 +1033,7 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restr
 
 // The same for the gated product: columns 32b .. 32b+15 of the partial sums are gates, 32b+16 .. 32b+31 the ups of
 // outputs 16b .. 16b+15; the output [M, N/2] is silu(gate) * up in bfloat16.
-__global__ void skinny_reduce_gated_kernel(const float* __restrict__ P, bf16_t* __restrict__ C, int M, int N, int splits, long ldc) {
+__global__ void skinny_reduce_gated_kernel(const float* __restrict__ P, bf16_t* __restrict__ C, int M, int N, int splits, long ldc, int gelu) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int half = N / 2;
     if (i >= (size_t)M * half) return;
@@ -1031,7 +1044,7 @@ __global__ void skinny_reduce_gated_kernel(const float* __restrict__ P, bf16_t* 
         gate += P[((size_t)sp * M + m) * N + col];
         up += P[((size_t)sp * M + m) * N + col + 16];
     }
-    C[m * ldc + c] = f32_to_bf16(silu_gate(gate, up));
+    C[m * ldc + c] = f32_to_bf16(gelu ? gelu_gate(gate, up) : silu_gate(gate, up));
 }
 
 // The same for the q/k/v product of an attention layer, N = (n_heads + 2 n_kv) * hd columns: the sums of a row are its queries,
@@ -1244,7 +1257,7 @@ __global__ __launch_bounds__(512, 4) void gemm_bf16_slim_kernel(const bf16_t* __
     __syncthreads();
     // Element v of a lane's result: activation row 4*q + v, weight row r of the strip (folded: of the group's 8 rows, and the
     // second half of k at row + 8, weight row + 8).
-    if (tid < 256 * (EPI == EPI_GATED_BF16 ? 1 : STRIPS)) {
+    if (tid < 256 * (is_gated(EPI) ? 1 : STRIPS)) {
         const int st = tid >> 8, e = tid & 255, m = e >> 4, c = e & 15;
         const int group = FOLD ? m >> 3 : 0, m_in = FOLD ? m & 7 : m;
         const int src_lane = c + 16 * (m_in >> 2), v = m_in & 3;
@@ -1252,7 +1265,7 @@ __global__ __launch_bounds__(512, 4) void gemm_bf16_slim_kernel(const bf16_t* __
         if constexpr (HAND) r = norm_in.squares != nullptr ? row_scale[m] : 1.0f;
         float square = 0.f;
         if (m < M && c < ROWS && group < XT) {
-            if constexpr (EPI == EPI_GATED_BF16) {
+            if constexpr (is_gated(EPI)) {
                 float gate = 0.f, up = 0.f;
 #pragma unroll
                 for (int s = 0; s < SLICES; ++s) {
@@ -1260,7 +1273,7 @@ __global__ __launch_bounds__(512, 4) void gemm_bf16_slim_kernel(const bf16_t* __
                     up += red[s * STRIPS + 1][0][src_lane][v];
                 }
                 if constexpr (HAND) { gate *= r; up *= r; }
-                ((bf16_t*)C)[(size_t)m * ldc + blockIdx.x * 16 + c] = f32_to_bf16(silu_gate(gate, up));
+                ((bf16_t*)C)[(size_t)m * ldc + blockIdx.x * 16 + c] = f32_to_bf16(gate_of<EPI>(gate, up));
             } else {
                 float sum = 0.f;
 #pragma unroll
@@ -1462,9 +1475,9 @@ static const NormOut NO_NORM_OUT = {nullptr, nullptr, 0, nullptr};
 
 static int reduce_partials(const float* scratch, void* C, int epi, int M, int N, int splits, long ldc, hipStream_t stream, NormIn norm_in = NO_NORM_IN,
                            NormOut norm_out = NO_NORM_OUT) {
-    if (epi == EPI_GATED_BF16) {
+    if (is_gated(epi)) {
         GI_REQUIRE(norm_in.squares == nullptr, "gemm_bf16: a gated product whose k is shared out cannot finish a norm handed on");
-        skinny_reduce_gated_kernel<<<(unsigned)(((size_t)M * (N / 2) + 255) / 256), 256, 0, stream>>>(scratch, (bf16_t*)C, M, N, splits, ldc);
+        skinny_reduce_gated_kernel<<<(unsigned)(((size_t)M * (N / 2) + 255) / 256), 256, 0, stream>>>(scratch, (bf16_t*)C, M, N, splits, ldc, epi == EPI_GATED_GELU_BF16 ? 1 : 0);
     } else {
 #define REDUCE(VEC_)                                                                                                                    \
     do {                                                                                                                                \
@@ -1539,9 +1552,9 @@ static int launch_slim(const void* A, const void* W, void* C, int epi, int M, in
         if (hand) gemm_bf16_slim_kernel<STRIPS_, ROWS_, EPI_, true><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, norm_in, norm_out); \
         else gemm_bf16_slim_kernel<STRIPS_, ROWS_, EPI_, false><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, norm_in, norm_out);     \
     } while (0)
-    if (epi == EPI_GATED_BF16) {
+    if (is_gated(epi)) {
         dim3 grid(N / 32);
-        SLIM(2, 16, EPI_GATED_BF16);
+        if (epi == EPI_GATED_BF16) SLIM(2, 16, EPI_GATED_BF16); else SLIM(2, 16, EPI_GATED_GELU_BF16);
     } else if (slim_strip_rows(M, N, epi) == 16) {
         dim3 grid((N + 15) / 16);
         if (epi == EPI_STORE_F32) SLIM(1, 16, EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM(1, 16, EPI_ADD_F32); else SLIM(1, 16, EPI_STORE_BF16);
@@ -1578,7 +1591,7 @@ static int launch_slim(const void* A, const void* W, void* C, int epi, int M, in
 // second grid dimension: 256 workgroups at 64 rows and N = 2048, each with 64 KB of weights and its own 128 KB of A) measured
 // equal at 33 to 64 rows and 3 % slower in the whole step from 65 rows on: not kept.
 static bool takes_slim_tiles(int M, int N, int K, int epi) {
-    return !takes_slim(M, N, K) && M <= 32 && K <= 2048 && epi != EPI_GATED_BF16 && gi_gemm_bf16_skinny_splits(N, K) > 0;
+    return !takes_slim(M, N, K) && M <= 32 && K <= 2048 && !is_gated(epi) && gi_gemm_bf16_skinny_splits(N, K) > 0;
 }
 
 // Weight rows per workgroup of that kernel: 16, or 12 or 8 where strips of 16 fill the compute units unevenly and those fill
@@ -1634,7 +1647,7 @@ static int launch_skinny(const void* A, const void* W, void* C, int epi, int M, 
         GI_REQUIRE(norm_out.scaled == nullptr && rope == nullptr, "gemm_bf16: a product this wide does not hand a norm on, or its rows to the cache");
         const int k_per_split = K;
         dim3 grid((N + 63) / 64, 1);
-        if (epi == EPI_GATED_BF16) SKINNY_MT(EPI_GATED_BF16, false); else if (epi == EPI_STORE_F32) SKINNY_MT(EPI_STORE_F32, false);
+        if (epi == EPI_GATED_BF16) SKINNY_MT(EPI_GATED_BF16, false); else if (epi == EPI_GATED_GELU_BF16) SKINNY_MT(EPI_GATED_GELU_BF16, false); else if (epi == EPI_STORE_F32) SKINNY_MT(EPI_STORE_F32, false);
         else if (epi == EPI_ADD_F32) SKINNY_MT(EPI_ADD_F32, false); else SKINNY_MT(EPI_STORE_BF16, false);
         GI_CHECK_LAUNCH("gemm_bf16 (skinny)");
         return 0;
@@ -1689,7 +1702,8 @@ static int launch_large(const void* A, const void* W, void* C, int epi, int M, i
         else if (epi == EPI_STORE_F32) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_STORE_F32, C, ldc, 1, K, 0L, NO_NORM_IN, NO_ROPE);            \
         else if (epi == EPI_ADD_F32) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_ADD_F32, C, ldc, 1, K, 0L, NO_NORM_IN, NO_ROPE);                \
         else if (epi == EPI_STORE_BF16) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_STORE_BF16, C, ldc, 1, K, 0L, NO_NORM_IN, NO_ROPE);          \
-        else PIPED(BM_, BN_, WM_, WN_, ST_, EPI_GATED_BF16, C, ldc, 1, K, 0L, NO_NORM_IN, NO_ROPE);                                     \
+        else if (epi == EPI_GATED_BF16) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_GATED_BF16, C, ldc, 1, K, 0L, NO_NORM_IN, NO_ROPE);          \
+        else PIPED(BM_, BN_, WM_, WN_, ST_, EPI_GATED_GELU_BF16, C, ldc, 1, K, 0L, NO_NORM_IN, NO_ROPE);                                \
     } while (0)
     const int splits = gi_gemm_bf16_piped_splits(M, N, K);
     if (splits > 1) {                              // few tiles: k is shared out, the sums are finished by the reduce kernel
@@ -1710,7 +1724,7 @@ static int launch_large(const void* A, const void* W, void* C, int epi, int M, i
     // workgroups per unit with two stages each when there are enough tiles, else one workgroup of eight waves with four stages.
     const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
     GI_REQUIRE(norm_out.scaled == nullptr || (!takes_pingpong(M, N) && large_norm_parts(M, N, K) > 0), "gemm_bf16: a product of M %d, N %d, K %d hands no norm on", M, N, K);
-    GI_REQUIRE(norm_in.squares == nullptr || rope != nullptr || (epi == EPI_GATED_BF16 && takes_pingpong(M, N) && norm_in.parts <= PIPED_MAX_PARTS),
+    GI_REQUIRE(norm_in.squares == nullptr || rope != nullptr || (is_gated(epi) && takes_pingpong(M, N) && norm_in.parts <= PIPED_MAX_PARTS),
                "gemm_bf16: a product of M %d, N %d, K %d takes no norm handed on in %d pieces", M, N, K, norm_in.parts);
     if (takes_pingpong(M, N) && rope == nullptr) {     // 256 x 256 tiles for most of the compute units: the ping-pong kernel
 #define PINGPONG(EPI_)                                                                                                                  \
@@ -1727,7 +1741,7 @@ static int launch_large(const void* A, const void* W, void* C, int epi, int M, i
     } while (0)
         GI_REQUIRE(lda < (1L << 22) && ldw < (1L << 22), "gemm_bf16: row strides %ld, %ld are too large for the tile-relative addressing", lda, ldw);
         if (epi == EPI_STORE_F32) PINGPONG(EPI_STORE_F32); else if (epi == EPI_ADD_F32) PINGPONG(EPI_ADD_F32);
-        else if (epi == EPI_STORE_BF16) PINGPONG(EPI_STORE_BF16); else PINGPONG(EPI_GATED_BF16);
+        else if (epi == EPI_STORE_BF16) PINGPONG(EPI_STORE_BF16); else if (epi == EPI_GATED_BF16) PINGPONG(EPI_GATED_BF16); else PINGPONG(EPI_GATED_GELU_BF16);
 #undef PINGPONG
         GI_CHECK_LAUNCH("gemm_bf16 (pingpong)");
         return 0;
@@ -1783,7 +1797,7 @@ GI_API int gi_gemm_bf16_handing(const void* A, const void* W, void* C, int c_dty
     int epi = epilogue_of(c_dtype, accumulate);
     if (gated) {
         GI_REQUIRE(N % 32 == 0 && c_dtype == GI_BF16 && !accumulate, "gemm_bf16: the gated product needs N %% 32 == 0 and a bfloat16 output");
-        epi = EPI_GATED_BF16;
+        epi = gated == 2 ? EPI_GATED_GELU_BF16 : EPI_GATED_BF16;
     }
     GI_REQUIRE(epi >= 0, "gemm_bf16: output dtype %d with accumulate %d is not supported", c_dtype, accumulate);
     GI_REQUIRE(squares_in == nullptr || (parts_in > 0 && gi_gemm_bf16_takes_norm(M, N, K, gated)),
@@ -1864,7 +1878,7 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
     int epi = epilogue_of(c_dtype, accumulate);
     if (gated) {
         GI_REQUIRE(N % 32 == 0 && c_dtype == GI_BF16 && !accumulate, "gemm_bf16: the gated product needs N %% 32 == 0 and a bfloat16 output");
-        epi = EPI_GATED_BF16;
+        epi = gated == 2 ? EPI_GATED_GELU_BF16 : EPI_GATED_BF16;
     }
     GI_REQUIRE(epi >= 0, "gemm_bf16: output dtype %d with accumulate %d is not supported", c_dtype, accumulate);
 
@@ -1879,11 +1893,11 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
     if ((long)((M + 127) / 128) * ((N + BN - 1) / BN) < 512) {   // few tiles: smaller ones fill more of the chip
         dim3 grid((N + BN - 1) / BN, (M + 63) / 64);
         if (epi == EPI_STORE_F32) TILED(64, EPI_STORE_F32); else if (epi == EPI_ADD_F32) TILED(64, EPI_ADD_F32);
-        else if (epi == EPI_STORE_BF16) TILED(64, EPI_STORE_BF16); else TILED(64, EPI_GATED_BF16);
+        else if (epi == EPI_STORE_BF16) TILED(64, EPI_STORE_BF16); else if (epi == EPI_GATED_BF16) TILED(64, EPI_GATED_BF16); else TILED(64, EPI_GATED_GELU_BF16);
     } else {
         dim3 grid((N + BN - 1) / BN, (M + 127) / 128);
         if (epi == EPI_STORE_F32) TILED(128, EPI_STORE_F32); else if (epi == EPI_ADD_F32) TILED(128, EPI_ADD_F32);
-        else if (epi == EPI_STORE_BF16) TILED(128, EPI_STORE_BF16); else TILED(128, EPI_GATED_BF16);
+        else if (epi == EPI_STORE_BF16) TILED(128, EPI_STORE_BF16); else if (epi == EPI_GATED_BF16) TILED(128, EPI_GATED_BF16); else TILED(128, EPI_GATED_GELU_BF16);
     }
 #undef TILED
     GI_CHECK_LAUNCH("gemm_bf16 (tiled)");

@@ -936,7 +936,8 @@ def gemm_bf16_takes_norm(m, n, k, gated=False) -> bool:
 
 def gemm_bf16(a, w, out, accumulate=False, gated=False, checked=False, norm_in=None, norm_out=None):
     """out (=|+=) a @ w.T with bfloat16 operands on the matrix cores, float32 sums.
-    gated: w is [gate; up] interleaved in groups of 16 rows and out = silu(a @ gate.T) * (a @ up.T), bfloat16 [m, n/2].
+    gated: w is [gate; up] interleaved in groups of 16 rows and out = act(a @ gate.T) * (a @ up.T), bfloat16 [m, n/2]; act is
+    SiLU (gated = True or "silu") or the tanh form of GELU (gated = "gelu_tanh").
 
     An RMS norm between two products of a few rows, without a kernel of its own:
     norm_out = (g, scaled, squares), with accumulate: beside out += a @ w.T, scaled = bfloat16(g * out) and squares
@@ -953,6 +954,9 @@ def gemm_bf16(a, w, out, accumulate=False, gated=False, checked=False, norm_in=N
         raise KernelError("gemm_bf16: operands must be bfloat16 with K and row strides multiples of 8, 16-byte aligned")
     n_scratch = _scratch_floats(m, n, k)                             # partial sums where k is split over workgroups
     scratch = torch.empty(n_scratch, dtype=torch.float32, device=a.device) if n_scratch else None
+    if gated and gated is not True and gated not in ACTIVATIONS:
+        raise KernelError(f"gemm: unknown activation {gated!r} of a gated product; known: {', '.join(ACTIVATIONS)}")
+    gate_code = 0 if not gated else 1 + (0 if gated is True else ACTIVATIONS[gated])        # 1: SiLU, 2: GELU (tanh form)
     if _profile is not None:
         _profile.note = (f"{n}x{k}{' gated' if gated else ''}", n * k * w.element_size())
     if norm_in is not None or norm_out is not None:
@@ -968,11 +972,11 @@ def gemm_bf16(a, w, out, accumulate=False, gated=False, checked=False, norm_in=N
                 raise KernelError("gemm: handing a norm on needs a product of a few rows that adds onto float32 rows, float32 weights of the norm, "
                                   "bfloat16 [m, n] for the scaled rows and float32 [m, gemm_bf16_norm_parts] for the sums of squares")
             _dev(g, scaled, squares_out)
-        _call("gi_gemm_bf16_handing", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm: out"), 1 if accumulate else 0, 1 if gated else 0,
+        _call("gi_gemm_bf16_handing", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm: out"), 1 if accumulate else 0, gate_code,
               m, n, k, a.stride(0), w.stride(0), out.stride(0), _ptr(scratch), n_scratch, _ptr(squares_in), squares_in.shape[1] if squares_in is not None else 0, float(eps),
               _ptr(g), _ptr(scaled), scaled.stride(0) if scaled is not None else 0, _ptr(squares_out), _stream())
         return out
-    _call("gi_gemm_bf16", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm: out"), 1 if accumulate else 0, 1 if gated else 0,
+    _call("gi_gemm_bf16", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm: out"), 1 if accumulate else 0, gate_code,
           m, n, k, a.stride(0), w.stride(0), out.stride(0), _ptr(scratch), n_scratch, _stream())
     return out
 

@@ -18,7 +18,8 @@ from .norm import HandedRows, NormedRows
 
 
 def linear(a, weight: torch.Tensor, out: torch.Tensor, accumulate: bool = False, gated: bool = False) -> torch.Tensor:
-    """gated: weight is [gate; up] interleaved by `ops.interleave_gate_up` and out = silu(gate) * up (bfloat16 only)."""
+    """gated: weight is [gate; up] interleaved by `ops.interleave_gate_up` and out = act(gate) * up (bfloat16 only); True or "silu"
+    for SiLU, "gelu_tanh" for the tanh form of GELU."""
     if isinstance(a, HandedRows):
         if (weight.dtype == torch.bfloat16 and ops.gemm_bf16_supports(a.scaled, weight, out)
                 and ops.gemm_bf16_takes_norm(a.scaled.shape[0], weight.shape[0], weight.shape[1], gated)):

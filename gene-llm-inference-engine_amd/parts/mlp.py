@@ -1,6 +1,6 @@
 """Gated feed-forward: residual += down( act(gate(h)) * up(h) ); act is SiLU, silu(g) = g / (1 + exp(-g))
 (SwiGLU; reference: src/model/transformer.cpp:437-450), or the tanh form of GELU where the spec says so.  gate and up run
-as one product with the stacked matrix [gate; up]; with SiLU and bfloat16 the gate is applied inside that product."""
+as one product with the stacked matrix [gate; up]; in bfloat16 the gate is applied inside that product."""
 from __future__ import annotations
 
 import torch
@@ -27,7 +27,7 @@ class SwiGlu(FeedForward):
         self.activation = getattr(spec, "activation", "silu")
         if self.activation not in ops.ACTIVATIONS:
             raise ValueError(f"feed-forward: unknown activation {self.activation!r}; known: {', '.join(ops.ACTIVATIONS)}")
-        self.fused = (self.activation == "silu" and self.in_dtype == torch.bfloat16 and self.mid_dtype == torch.bfloat16 and up.dtype == torch.bfloat16
+        self.fused = (self.in_dtype == torch.bfloat16 and self.mid_dtype == torch.bfloat16 and up.dtype == torch.bfloat16
                       and spec.intermediate_size % 16 == 0 and spec.hidden_size % 8 == 0)
         self.w_gate_up = ops.interleave_gate_up(gate, up) if self.fused else torch.cat([gate, up], dim=0).contiguous()
 
@@ -43,7 +43,7 @@ class SwiGlu(FeedForward):
         T, inter = ctx.n_rows, self.spec.intermediate_size
         if self.fused:
             mid = torch.empty((T, inter), dtype=torch.bfloat16, device=ctx.device)
-            linear(h, self.w_gate_up, mid, gated=True)
+            linear(h, self.w_gate_up, mid, gated=self.activation)
         else:
             gate_up = torch.empty((T, 2 * inter), dtype=torch.float32, device=ctx.device)
             linear(h, self.w_gate_up, gate_up)

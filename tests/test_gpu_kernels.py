@@ -106,6 +106,12 @@ def test_gemm_bf16_gated(m, inter, k):
     want = torch.nn.functional.silu(a.double() @ gate.double().T) * (a.double() @ up.double().T)
     assert rel(out[:, :inter], want) < 6e-3
     assert torch.all(out[:, inter:] == 3.0)
+    # the same product gated by the tanh form of GELU, stated here as 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))
+    ops().gemm_bf16(a, w, out[:, :inter], gated="gelu_tanh")
+    z = a.double() @ gate.double().T
+    want = 0.5 * z * (1 + torch.tanh((2 / torch.pi) ** 0.5 * (z + 0.044715 * z ** 3))) * (a.double() @ up.double().T)
+    assert rel(out[:, :inter], want) < 6e-3
+    assert torch.all(out[:, inter:] == 3.0)
 
 
 @pytest.mark.parametrize("m,n,k", [(4109, 4120, 192), (4096, 4096, 448)])
