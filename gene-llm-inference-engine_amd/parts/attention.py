@@ -19,6 +19,7 @@ from ..weights.loader import TensorNeed
 from .base import Mixer, PositionEncoding, position_class, register_mixer
 from .linear import activation_dtype_for, linear, linear_onto
 from .norm import HandedRows, NormedRows
+from .rope import rotation_tables
 
 
 def qkv_rotate_store_attend(h, w_qkv, ctx, cache, *, n_heads, n_kv_heads, head_dim, position=None, window=None, in_dtype=None,
@@ -161,7 +162,6 @@ class Attention(Mixer):
 
     def _attend_general(self, h, ctx, cache):
         """The heads' outputs [rows, heads * value_dim] by the general path."""
-        from .rope import rotation_tables
         s, T, vd = self.spec, ctx.n_rows, self.value_dim
         proj = torch.empty((T, self.w_qkv.shape[0]), dtype=torch.float32, device=ctx.device)
         linear(h, self.w_qkv, proj)

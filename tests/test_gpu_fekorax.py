@@ -435,3 +435,52 @@ def test_generation_from_the_command_line_on_random_weights(tmp_path):
     runs = [subprocess.run(cmd, capture_output=True, text=True, timeout=280) for _ in range(2)]
     assert all(r.returncode == 0 for r in runs), runs[0].stderr[-2000:]
     assert runs[0].stdout == runs[1].stdout and len(runs[0].stdout.split()) >= 20
+
+
+def test_the_new_parts_serve_other_designs():
+    """The parts are not Fekorax's own: a model put together by hand, one sandwich layer around the plain attention of a Llama layer
+    and a SiLU-gated feed-forward, one pre-norm layer around a matrix memory and a GELU-gated feed-forward, through the same step
+    function; against a plain computation from the two plain implementations' functions."""
+    from geneinfer_amd.config import AttentionSpec, LayerSpec, MlstmSpec, ModelSpec, RmsNormSpec, RotarySpec, RunEntry, SwiGluSpec
+    from geneinfer_amd.engine import Runner
+    from geneinfer_amd.engine.model import DecoderModel
+    from geneinfer_amd.parts import model_tensor_needs
+    from geneinfer_amd.weights import random_tensors
+    from plain_fekorax import capped
+    from plain_llama import causal_attention, rms_norm, rope_inverse_frequencies, rope_rotate, swiglu
+    d, vocab, eps = 64, 100, 1e-5
+    norm = lambda name: RmsNormSpec(d, eps, name)
+    spec = ModelSpec(architecture="by hand", vocab_size=vocab, hidden_size=d, max_positions=256, embedding="emb", final_norm=norm("fn"), lm_head="head", layers=(
+        LayerSpec(mixer=AttentionSpec(d, 4, 2, 16, "a.q", "a.k", "a.v", "a.o", RotarySpec(16, 10000.0)), feed_forward=SwiGluSpec(d, 96, "f.g", "f.u", "f.d"),
+                  mixer_norm=norm("n1"), feed_forward_norm=norm("n2"), block="sandwich", mixer_post_norm=norm("n1b"), feed_forward_post_norm=norm("n2b")),
+        LayerSpec(mixer=MlstmSpec(d, 2, 8, 24, 7.0, eps, "m.q", "m.k", "m.v", "m.g", "m.o", "m.n", "m.i", "m.ib", "m.f", "m.fb"),
+                  feed_forward=SwiGluSpec(d, 80, "g.g", "g.u", "g.d", activation="gelu_tanh"), mixer_norm=norm("p1"), feed_forward_norm=norm("p2"), block="prenorm")),
+        run_order=(RunEntry(0), RunEntry(1)))
+    host = random_tensors(model_tensor_needs(spec), seed=5, dtype="float32", std=0.2)
+    model = DecoderModel(spec, {k: v.to(DEV) for k, v in host.items()}, torch.float32, DEV)
+    runner = Runner(model, page_size=4, max_tokens=256, max_requests=2)
+    tokens = _prompt(dict(vocab=vocab), 45, 2)
+    got = {}
+    for what, cuts in (("whole", [45]), ("cut", [3, 20, 2])):
+        runner.open(what)
+        got[what] = feed(runner, what, tokens, cuts)
+        runner.close(what)
+    assert torch.equal(got["whole"], got["cut"])
+
+    w = {k: v.double() for k, v in host.items()}
+    T, pos = len(tokens), torch.arange(len(tokens))
+    x = w["emb"][torch.tensor(tokens)]
+    h = rms_norm(x, w["n1"], eps)
+    f = rope_inverse_frequencies(16, 10000.0)
+    q, k = rope_rotate((h @ w["a.q"].T).view(T, 4, 16), pos, f), rope_rotate((h @ w["a.k"].T).view(T, 2, 16), pos, f)
+    y = causal_attention(q, k, (h @ w["a.v"].T).view(T, 2, 16)).reshape(T, 64) @ w["a.o"].T
+    x = x + rms_norm(y, w["n1b"], eps)
+    x = x + rms_norm(swiglu(rms_norm(x, w["n2"], eps), w["f.g"], w["f.u"], w["f.d"]), w["n2b"], eps)
+    h = rms_norm(x, w["p1"], eps)
+    o = matrix_memory((h @ w["m.q"].T).view(T, 2, 8) * 8 ** -0.5, (h @ w["m.k"].T).view(T, 2, 8), (h @ w["m.v"].T).view(T, 2, 24),
+                      capped(h @ w["m.i"].T + w["m.ib"], 7.0), torch.nn.functional.logsigmoid(capped(h @ w["m.f"].T + w["m.fb"], 7.0)))
+    x = x + (unit_rms(o, eps).reshape(T, 48) * w["m.n"] * torch.sigmoid(h @ w["m.g"].T)) @ w["m.o"].T
+    h = rms_norm(x, w["p2"], eps)
+    x = x + (gelu_tanh(h @ w["g.g"].T) * (h @ w["g.u"].T)) @ w["g.d"].T
+    want = rms_norm(x, w["fn"], eps) @ w["head"].T
+    assert relative_error(got["whole"], want) < 5e-5
