@@ -70,7 +70,7 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(const float* __restrict_
                                                        const float* __restrict__ i_bias, const float* __restrict__ f_bias, float cap, float q_scale,
                                                        const int* __restrict__ seg_start, const int* __restrict__ seg_len,
                                                        const int* __restrict__ row_slot, float* __restrict__ state, long state_stride,
-                                                       float* __restrict__ out, long ldo, int dk, int dv) {
+                                                       float* __restrict__ out, long ldo, float* __restrict__ den, int dk, int dv) {
     constexpr int C = 4, VC = 3;                 // columns a wave holds: three of S and n (as the column of a value that is always 1)
     constexpr int RG = 64 / C;                   // groups of rows: lane = column * RG + group, so that a column's groups are neighbouring lanes
     constexpr int KQ = RG * ROWS;                // rows a token's k and q cover (dk, padded with zeros)
@@ -160,10 +160,14 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(const float* __restrict_
                 }
             };
             // The groups' shares are added by lane moves; n . q is then in the last column's lanes, the same for the whole wave.
+            // The columns' sums leave undivided; what they are to be divided by, max(|n . q|, exp(-m)) + 1e-6, one number per
+            // token and head, is written by the head's first tile, and whoever reads the sums divides (the kernel behind this
+            // one reads every sum once anyway; a division per token in every wave is a sixth of what a wave does here).
             auto finish = [&](int u, float acc, float floor_) {
                 acc = group_sum<RG>(acc);
-                const float x = fmaxf(fabsf(lane_value(acc, VC * RG)), floor_) + 1e-6f;
-                if (rg == 0 && live) out[(size_t)(t0 + b0 + s0 + u) * ldo + h * dv + col] = acc / x;
+                const size_t t = (size_t)(t0 + b0 + s0 + u);
+                if (rg == 0 && live) out[t * ldo + h * dv + col] = acc;
+                if (vt == 0 && lane == VC * RG) den[t * gridDim.y + h] = fmaxf(fabsf(acc), floor_) + 1e-6f;
             };
             constexpr int UB = TB >= 4 ? 4 : TB;     // so many tokens at a time, so that their reads of LDS go out together
             int u = 0;
@@ -193,17 +197,24 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(const float* __restrict_
 }
 
 // y[t, h*dv + d] = w[h*dv + d] * o[t, h, d] * rsqrt(mean_d(o[t, h, :]^2) + eps) * sigmoid(g[t, h*dv + d]): one wave per (row, head).
+// With `den` [rows, heads], o is what the rows hold divided by den[t, h] (the matrix memory's sums and their divisor).
 template <typename TW, typename TO>
-__global__ __launch_bounds__(64) void head_norm_gate_kernel(const float* __restrict__ o, long ldo, const float* __restrict__ g, long ldg,
-                                                           const TW* __restrict__ w, TO* __restrict__ y, long ldy, int n_heads, int dv, float eps) {
+__global__ __launch_bounds__(64) void head_norm_gate_kernel(const float* __restrict__ o, long ldo, const float* __restrict__ den,
+                                                           const float* __restrict__ g, long ldg, const TW* __restrict__ w,
+                                                           TO* __restrict__ y, long ldy, int n_heads, int dv, float eps) {
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const float* orow = o + (size_t)t * ldo + (size_t)h * dv;
+    const float by = den ? den[(size_t)t * n_heads + h] : 1.0f;
     float ss = 0.f;
-    for (int d = lane; d < dv; d += 64) ss = fmaf(orow[d], orow[d], ss);
+    for (int d = lane; d < dv; d += 64) {
+        const float v = den ? orow[d] / by : orow[d];
+        ss = fmaf(v, v, ss);
+    }
     const float r = 1.0f / sqrtf(wave_sum(ss) / (float)dv + eps);
     for (int d = lane; d < dv; d += 64) {
+        const float v = den ? orow[d] / by : orow[d];
         const float gate = 1.0f / (1.0f + expf(-g[(size_t)t * ldg + (size_t)h * dv + d]));
-        store_f32(y, (size_t)t * ldy + (size_t)h * dv + d, load_f32(w, (size_t)h * dv + d) * (orow[d] * r) * gate);
+        store_f32(y, (size_t)t * ldy + (size_t)h * dv + d, load_f32(w, (size_t)h * dv + d) * (v * r) * gate);
     }
 }
 
@@ -224,28 +235,30 @@ GI_API long gi_mlstm_state_floats(int n_heads, int dk, int dv) {
 GI_API int gi_mlstm_max_key_dim() { return 512; }
 
 // proj: float32 [n_rows, ld], whose columns q_off.. hold q [heads*dk], k_off.. k [heads*dk], v_off.. v [heads*dv], i_off.. and
-// f_off.. the gates' pre-activations [heads]; out: float32 [n_rows, ldo] gets o [heads*dv]; state: [slots, state_stride].
+// f_off.. the gates' pre-activations [heads]; out: float32 [n_rows, ldo] gets the heads' sums S^T q [heads*dv], den: float32
+// [n_rows, heads] what each head's sums are to be divided by (o = out / den); state: [slots, state_stride].
 GI_API int gi_mlstm_scan(const float* proj, long ld, int q_off, int k_off, int v_off, int i_off, int f_off, const float* i_bias, const float* f_bias,
                          float cap, float q_scale, const int* seg_start, const int* seg_len, int n_segs, const int* row_slot, float* state,
-                         long state_stride, float* out, long ldo, int n_heads, int dk, int dv, hipStream_t stream) {
+                         long state_stride, float* out, long ldo, float* den, int n_heads, int dk, int dv, hipStream_t stream) {
+    GI_REQUIRE(den != nullptr, "mlstm_scan: the divisors need a place");
     GI_REQUIRE(n_segs > 0 && n_heads > 0 && dk > 0 && dk <= 512 && dv > 0, "mlstm_scan: bad sizes (runs %d, heads %d, dk %d, dv %d; dk at most 512)", n_segs, n_heads, dk, dv);
     GI_REQUIRE(cap > 0.f && state_stride >= gi_mlstm_state_floats(n_heads, dk, dv) && ldo >= (long)n_heads * dv, "mlstm_scan: bad cap, state stride or output stride");
     const int tiles = (dv + 2) / 3;
     GI_REQUIRE(n_heads <= 65535 && tiles <= 65535, "mlstm_scan: too many heads or value channels");
     dim3 grid(n_segs, n_heads, tiles);
 #define GO(R) mlstm_scan_kernel<R><<<grid, 64, 0, stream>>>(proj, ld, q_off, k_off, v_off, i_off, f_off, i_bias, f_bias, cap, q_scale, seg_start, seg_len, \
-                                                           row_slot, state, state_stride, out, ldo, dk, dv)
+                                                           row_slot, state, state_stride, out, ldo, den, dk, dv)
     if (dk <= 64) GO(4); else if (dk <= 128) GO(8); else if (dk <= 256) GO(16); else GO(32);
 #undef GO
     GI_CHECK_LAUNCH("mlstm_scan");
     return 0;
 }
 
-GI_API int gi_head_norm_gate(const float* o, long ldo, const float* g, long ldg, const void* w, int w_dtype, void* y, int y_dtype, long ldy, int n_rows,
+GI_API int gi_head_norm_gate(const float* o, long ldo, const float* den, const float* g, long ldg, const void* w, int w_dtype, void* y, int y_dtype, long ldy, int n_rows,
                              int n_heads, int dv, float eps, hipStream_t stream) {
     GI_REQUIRE(n_rows > 0 && n_heads > 0 && n_heads <= 65535 && dv > 0, "head_norm_gate: bad sizes (rows %d, heads %d, dv %d)", n_rows, n_heads, dv);
     dim3 grid(n_rows, n_heads);
-#define GO(TW, TO) head_norm_gate_kernel<TW, TO><<<grid, 64, 0, stream>>>(o, ldo, g, ldg, (const TW*)w, (TO*)y, ldy, n_heads, dv, eps)
+#define GO(TW, TO) head_norm_gate_kernel<TW, TO><<<grid, 64, 0, stream>>>(o, ldo, den, g, ldg, (const TW*)w, (TO*)y, ldy, n_heads, dv, eps)
     if (w_dtype == GI_F32 && y_dtype == GI_F32) GO(float, float);
     else if (w_dtype == GI_F32 && y_dtype == GI_BF16) GO(float, bf16_t);
     else if (w_dtype == GI_BF16 && y_dtype == GI_BF16) GO(bf16_t, bf16_t);

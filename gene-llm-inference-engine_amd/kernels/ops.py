@@ -43,8 +43,8 @@ _SIGNATURES = {
     "gi_act_mul": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "gi_segments": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p],
     "gi_mlstm_scan": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_int, c_void_p,
-                      c_void_p, c_long, c_void_p, c_long, c_int, c_int, c_int, c_void_p],
-    "gi_head_norm_gate": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_float, c_void_p],
+                      c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_void_p],
+    "gi_head_norm_gate": [c_void_p, c_long, c_void_p, c_void_p, c_long, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_float, c_void_p],
     "gi_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long, c_void_p],
     "gi_attention_prompt_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
                                  c_float, c_int, c_void_p, c_void_p, c_int, c_void_p, c_long, c_int, c_void_p, c_void_p, c_long, c_void_p],
@@ -552,11 +552,15 @@ def mlstm_max_key_dim() -> int:
     return MLSTM_MAX_KEY_DIM
 
 
-def mlstm_scan(proj, offsets, i_bias, f_bias, cap, q_scale, seg_start, seg_len, row_slot, state, out, n_heads, dk, dv):
+def mlstm_scan(proj, offsets, i_bias, f_bias, cap, q_scale, seg_start, seg_len, row_slot, state, out, den, n_heads, dk, dv):
     """The matrix memories of a step's requests stepped over the requests' rows, in order (csrc/recurrent.hip states the recurrence).
-    proj: float32 [n, columns]; offsets = the first columns of (q, k, v, i, f) in it; out: float32 [n, heads*dv];
-    state: float32 [slots, mlstm_state_floats], read at each request's first row of the step and written after its last."""
-    _dev(proj, i_bias, f_bias, seg_start, seg_len, row_slot, state, out)
+    proj: float32 [n, columns]; offsets = the first columns of (q, k, v, i, f) in it; out: float32 [n, heads*dv] gets the heads'
+    sums S^T q and den: float32 [n, heads] what each head's are to be divided by (the readout is out / den: `head_norm_gate`
+    divides on its way); state: float32 [slots, mlstm_state_floats], read at each request's first row of the step and written
+    after its last."""
+    _dev(proj, i_bias, f_bias, seg_start, seg_len, row_slot, state, out, den)
+    if not (den.dtype == torch.float32 and den.shape == (proj.shape[0], n_heads) and den.is_contiguous()):
+        raise KernelError("mlstm_scan: den must be float32 [n, heads], contiguous")
     n = proj.shape[0]
     q_off, k_off, v_off, i_off, f_off = (int(o) for o in offsets)
     if not (proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and out.dtype == torch.float32 and out.shape == (n, n_heads * dv) and out.stride(1) == 1):
@@ -574,21 +578,24 @@ def mlstm_scan(proj, offsets, i_bias, f_bias, cap, q_scale, seg_start, seg_len, 
         raise KernelError("mlstm_scan: state must be float32 [slots, mlstm_state_floats]")
     _call("gi_mlstm_scan", proj.data_ptr(), proj.stride(0), q_off, k_off, v_off, i_off, f_off, i_bias.data_ptr(), f_bias.data_ptr(), float(cap), float(q_scale),
           seg_start.data_ptr(), seg_len.data_ptr(), n_segs, row_slot.data_ptr(), state.data_ptr(), state.stride(0), out.data_ptr(), out.stride(0),
-          n_heads, dk, dv, _stream())
+          den.data_ptr(), n_heads, dk, dv, _stream())
     return out
 
 
-def head_norm_gate(o, gate, weight, eps, out, n_heads, dv):
+def head_norm_gate(o, gate, weight, eps, out, n_heads, dv, den=None):
     """out[t, h*dv + d] = weight[h*dv + d] * o[t, h, d] * rsqrt(mean over d of o[t, h, :]^2 + eps) * sigmoid(gate[t, h*dv + d]);
-    o and gate float32 [n, heads*dv] (unit inner stride: columns of a wider product are fine)."""
-    _dev(o, gate, weight, out)
+    o and gate float32 [n, heads*dv] (unit inner stride: columns of a wider product are fine).  den: float32 [n, heads]; o is
+    then what the rows hold divided by den[t, h]."""
+    _dev(o, gate, weight, out, den)
     n = o.shape[0]
+    if den is not None and not (den.dtype == torch.float32 and den.shape == (n, n_heads) and den.is_contiguous()):
+        raise KernelError("head_norm_gate: den must be float32 [n, heads], contiguous")
     for t, name in ((o, "o"), (gate, "gate")):
         if not (t.dtype == torch.float32 and t.shape == (n, n_heads * dv) and t.stride(1) == 1):
             raise KernelError(f"head_norm_gate: {name} must be float32 [n, heads*dv]")
     if not (weight.numel() == n_heads * dv and weight.is_contiguous() and out.shape == (n, n_heads * dv) and out.stride(1) == 1):
         raise KernelError("head_norm_gate: weight must be [heads*dv] and out [n, heads*dv]")
-    _call("gi_head_norm_gate", o.data_ptr(), o.stride(0), gate.data_ptr(), gate.stride(0), weight.data_ptr(), _code(weight, "head_norm_gate: weight"),
+    _call("gi_head_norm_gate", o.data_ptr(), o.stride(0), _ptr(den), gate.data_ptr(), gate.stride(0), weight.data_ptr(), _code(weight, "head_norm_gate: weight"),
           out.data_ptr(), _code(out, "head_norm_gate: out"), out.stride(0), n, n_heads, dv, float(eps), _stream())
     return out
 

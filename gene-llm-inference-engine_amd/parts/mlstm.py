@@ -60,11 +60,12 @@ class Mlstm(Mixer):
         proj = torch.empty((T, self.w_in.shape[0]), dtype=torch.float32, device=ctx.device)
         linear(h, self.w_in, proj)
         seg_start, seg_len = ops.segments(ctx)
-        heads_out = torch.empty((T, vv), dtype=torch.float32, device=ctx.device)
+        sums = torch.empty((T, vv), dtype=torch.float32, device=ctx.device)          # the heads' S^T q, and what to divide them by
+        divisors = torch.empty((T, s.n_heads), dtype=torch.float32, device=ctx.device)
         ops.mlstm_scan(proj, (o["q"], o["k"], o["v"], o["i"], o["f"]), self.i_bias, self.f_bias, s.gate_cap, s.key_dim ** -0.5, seg_start, seg_len,
-                       ctx.row_slot, cache.state, heads_out, s.n_heads, s.key_dim, s.value_dim)
+                       ctx.row_slot, cache.state, sums, divisors, s.n_heads, s.key_dim, s.value_dim)
         mid = torch.empty((T, vv), dtype=self.mid_dtype, device=ctx.device)
-        ops.head_norm_gate(heads_out, proj[:, o["g"]:o["g"] + vv], self.out_norm, s.norm_eps, mid, s.n_heads, s.value_dim)
+        ops.head_norm_gate(sums, proj[:, o["g"]:o["g"] + vv], self.out_norm, s.norm_eps, mid, s.n_heads, s.value_dim, den=divisors)
         if overwrite:
             linear(mid, self.w_o, residual)
         else:

@@ -120,11 +120,11 @@ def test_matrix_memory_kernel(heads, dk, dv):
 
     def run(rows, seg_lens, slots):
         starts = [sum(seg_lens[:i]) for i in range(len(seg_lens))]
-        out = torch.empty(rows.shape[0], heads * dv, device=DEV)
+        out, den = torch.empty(rows.shape[0], heads * dv, device=DEV), torch.empty(rows.shape[0], heads, device=DEV)
         row_slot = torch.tensor([s for s, n in zip(slots, seg_lens) for _ in range(n)], dtype=torch.int32, device=DEV)
         ops.mlstm_scan(dev(rows), off, dev(i_b), dev(f_b), cap, dk ** -0.5, torch.tensor(starts, dtype=torch.int32, device=DEV),
-                       torch.tensor(seg_lens, dtype=torch.int32, device=DEV), row_slot, state, out, heads, dk, dv)
-        return out.cpu().double()
+                       torch.tensor(seg_lens, dtype=torch.int32, device=DEV), row_slot, state, out, den, heads, dk, dv)
+        return (out.view(-1, heads, dv) / den[:, :, None]).reshape(-1, heads * dv).cpu().double()       # (the kernel leaves the division to its reader)
 
     got = run(proj, lens, [2, 0])
     assert relative_error(got, want) < 2e-5
