@@ -19,11 +19,13 @@ from typing import Any, ClassVar, Optional, Tuple
 class RotarySpec:
     """Rotation of the pairs (k, k + head_dim/2) of every head by pos * f_k, with f_k = theta^(-2k/head_dim) unless the
     architecture gives its own `frequencies` (head_dim/2 numbers: whatever rule stretches or blends them is the
-    architecture's, applied where it builds this spec)."""
+    architecture's, applied where it builds this spec).  `magnitude` multiplies every cosine and sine (rules that stretch the
+    frequencies for longer contexts may lengthen the turned vectors a little)."""
     kind: ClassVar[str] = "rotary_half_split"
     head_dim: int
     theta: float
     frequencies: Optional[Tuple[float, ...]] = None
+    magnitude: float = 1.0
 
     def __post_init__(self):
         if self.frequencies is not None and len(self.frequencies) != self.head_dim // 2:
@@ -33,16 +35,36 @@ class RotarySpec:
 @dataclass(frozen=True)
 class PartialRotarySpec:
     """Rotation of the pairs (k, k + rotary_dim/2) of the first `rotary_dim` channels of every head by pos * f_k; the other
-    channels of the head pass unchanged.  f_k = theta^(-2k/rotary_dim) unless the architecture gives its own `frequencies`."""
+    channels of the head pass unchanged.  f_k = theta^(-2k/rotary_dim) unless the architecture gives its own `frequencies`;
+    `magnitude` multiplies every cosine and sine."""
     kind: ClassVar[str] = "rotary_partial"
     head_dim: int
     rotary_dim: int
     theta: float
     frequencies: Optional[Tuple[float, ...]] = None
+    magnitude: float = 1.0
 
     def __post_init__(self):
         if self.rotary_dim % 2 or not 0 < self.rotary_dim <= self.head_dim:
             raise ValueError(f"a rotation of {self.rotary_dim} of a head's {self.head_dim} channels: an even number within the head is needed")
+        if self.frequencies is not None and len(self.frequencies) != self.rotary_dim // 2:
+            raise ValueError(f"a rotation of {self.rotary_dim} channels needs {self.rotary_dim // 2} frequencies, not {len(self.frequencies)}")
+
+
+@dataclass(frozen=True)
+class InterleavedRotarySpec:
+    """Rotation of the neighbouring pairs (2k, 2k + 1) of `rotary_dim` channels by pos * f_k, f_k = theta^(-2k/rotary_dim) unless
+    the architecture gives its own `frequencies`.  It only makes the cosines and sines; the mixer that names it says which
+    channels they turn."""
+    kind: ClassVar[str] = "rotary_interleaved"
+    rotary_dim: int
+    theta: float
+    frequencies: Optional[Tuple[float, ...]] = None
+    magnitude: float = 1.0
+
+    def __post_init__(self):
+        if self.rotary_dim % 2 or self.rotary_dim <= 0:
+            raise ValueError(f"a rotation of pairs needs an even number of channels, not {self.rotary_dim}")
         if self.frequencies is not None and len(self.frequencies) != self.rotary_dim // 2:
             raise ValueError(f"a rotation of {self.rotary_dim} channels needs {self.rotary_dim // 2} frequencies, not {len(self.frequencies)}")
 
@@ -79,6 +101,42 @@ class AttentionSpec:
     qk_norm_eps: float = 1e-6
     head_gate: Optional[str] = None  # tensor [heads, hidden]: head h's output is multiplied by sigmoid(row h of it . the mixer's input)
     keep_chunk: Optional[int] = None # the pages of chunks gone by are given back: set where this entry and every reader of its pages cut their masks alike
+    q_bias: Optional[str] = None     # tensors [heads*head_dim], [kv_heads*head_dim], [kv_heads*value_dim]: added to the projections
+    k_bias: Optional[str] = None
+    v_bias: Optional[str] = None
+    # Values blended across layers: the layers that name one `value_family` share the values of the family's first layer in
+    # the run order (the one without `value_blend`); each other one caches and attends over (1 - w) v + w v_first, with w the
+    # number in its tensor `value_blend` and v_first the first layer's values of the same row.
+    value_family: Optional[str] = None
+    value_blend: Optional[str] = None
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Attention whose queries and keys/values pass through low-rank latents.  c_q = norm(W_dq x), q = W_uq c_q, per head
+    [head_dim unrotated | rotary_dim rotated]; W_dkv x = [kv_rank | rotary_dim]: the first part, normed, is the latent c, the
+    second one rotated key part for all heads; per head the unrotated key is W_uk c and the value W_uv c, so that only c and
+    the rotated part are cached.  score = (q_plain . k_plain + q_rot . k_rot) * scale; causal, optionally windowed."""
+    kind: ClassVar[str] = "latent_attention"
+    hidden_size: int
+    n_heads: int
+    head_dim: int                    # unrotated channels of a query/key head
+    rotary_dim: int                  # rotated channels
+    value_dim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    norm_eps: float
+    dq_proj: str
+    dq_norm: str
+    uq_proj: str
+    dkv_proj: str
+    dkv_norm: str
+    uk_proj: str
+    uv_proj: str
+    o_proj: str
+    position: Optional[Any] = None   # a spec that gives cosines and sines for rotary_dim / 2 neighbouring pairs
+    window: Optional[int] = None
 
 
 @dataclass(frozen=True)
@@ -91,6 +149,51 @@ class SwiGluSpec:
     up_proj: str
     down_proj: str
     activation: str = "silu"
+
+
+@dataclass(frozen=True)
+class DenseMlpSpec:
+    """down(act(up(x))), no gate, no biases.  `activation` "xielu": with the two numbers (p, q) of the tensor `activation_params`,
+    act(z) = softplus(p) z^2 + z/2 for z > 0 and (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2 otherwise."""
+    kind: ClassVar[str] = "dense_mlp"
+    hidden_size: int
+    intermediate_size: int
+    up_proj: str
+    down_proj: str
+    activation: str = "xielu"
+    activation_params: Optional[str] = None
+
+
+@dataclass(frozen=True)
+class GatedDeltaSpec:
+    """The gated delta rule: per head a memory S [key_dim, value_dim], zero at a sequence's start, and per token
+        S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q
+    with g = exp(-exp(a_log) softplus(a(x) + dt_bias)) and beta = sigmoid(b(x)) per head.  q and k (n_kv_heads heads, head h of
+    the memory uses q/k head h // (n_heads / n_kv_heads)) and v pass a causal convolution of `conv_taps` taps per channel
+    (tensors [channels, taps], the last tap the token's own) and SiLU; q and k are then divided by sqrt(sum of squares + 1e-6),
+    q also by sqrt(key_dim).  Every head's o is divided by its root mean square (`norm_eps`), multiplied by `out_norm`
+    [value_dim], one for all heads, and by SiLU(gate(x)), and goes through `o_proj`."""
+    kind: ClassVar[str] = "gated_delta"
+    hidden_size: int
+    n_heads: int
+    n_kv_heads: int
+    key_dim: int
+    value_dim: int
+    conv_taps: int
+    norm_eps: float
+    q_proj: str
+    k_proj: str
+    v_proj: str
+    q_conv: str
+    k_conv: str
+    v_conv: str
+    a_proj: str
+    a_log: str
+    dt_bias: str
+    b_proj: str
+    gate_proj: str
+    out_norm: str
+    o_proj: str
 
 
 @dataclass(frozen=True)

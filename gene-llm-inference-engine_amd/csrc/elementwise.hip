@@ -198,21 +198,22 @@ GI_API int gi_rmsnorm(const float* x, const int* rows, const void* w, int w_dtyp
 
 // -------------------------------------------------------------------------------- rotary angles
 // cos and sin of pos * f_k for every row, the angle taken in 64-bit: a 32-bit angle loses digits
-// at large positions (reference: src/kernels/kernels.cpp:145-161).
+// at large positions (reference: src/kernels/kernels.cpp:145-161).  `magnitude` multiplies both (1 for a plain rotation; rules
+// that stretch the frequencies for longer contexts lengthen the turned vectors a little as well).
 __global__ void rope_cos_sin_kernel(const int* __restrict__ pos, const double* __restrict__ inv_freq, float* __restrict__ cos_out,
-                                    float* __restrict__ sin_out, int n_rows, int half) {
+                                    float* __restrict__ sin_out, int n_rows, int half, float magnitude) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n_rows * half) return;
     const double a = (double)pos[i / half] * inv_freq[i % half];
-    cos_out[i] = (float)cos(a);
-    sin_out[i] = (float)sin(a);
+    cos_out[i] = (float)cos(a) * magnitude;
+    sin_out[i] = (float)sin(a) * magnitude;
 }
 
-GI_API int gi_rope_cos_sin(const int* pos, const double* inv_freq, float* cos_out, float* sin_out, int n_rows, int half,
+GI_API int gi_rope_cos_sin(const int* pos, const double* inv_freq, float* cos_out, float* sin_out, int n_rows, int half, float magnitude,
                            hipStream_t stream) {
     GI_REQUIRE(n_rows > 0 && half > 0, "rope_cos_sin: n_rows %d and half %d must be positive", n_rows, half);
     const int n = n_rows * half;
-    rope_cos_sin_kernel<<<(n + 255) / 256, 256, 0, stream>>>(pos, inv_freq, cos_out, sin_out, n_rows, half);
+    rope_cos_sin_kernel<<<(n + 255) / 256, 256, 0, stream>>>(pos, inv_freq, cos_out, sin_out, n_rows, half, magnitude);
     GI_CHECK_LAUNCH("rope_cos_sin");
     return 0;
 }
@@ -411,6 +412,10 @@ GI_API int gi_rmsnorm_add(const float* y, const void* w, int w_dtype, float* x, 
 //   (cos, sin: [n_rows, rot/2]; nullptr or rot = 0: no rotation); the other channels pass;
 //   queries go to q_out [n_rows, n_heads*hd]; keys to the page's [kv_head][place][hd]; values, of `vd` channels a head,
 //   to the page's [kv_head][vd][place] behind all keys.  k == nullptr: another layer's pages are read and none written.
+// Before any of that a projection's bias is added (q_bias [n_heads*hd], k_bias [n_kv*hd], v_bias [n_kv*vd], float32; nullptr: none).
+// Values may be blended with those another layer made of the same rows: with `v_other` [n_rows, ld_other] and `v_blend` (one
+// number on the device), v <- (1 - blend) v + blend v_other is what goes into the page; `v_keep` [n_rows, ld_keep], if given, gets
+// this layer's values (with their bias, before any blending) for such a reader.
 constexpr int NRS_MAX_HD = 512;
 
 template <typename TQ, typename TC, typename TW>
@@ -419,7 +424,10 @@ __global__ __launch_bounds__(64) void norm_rope_store_kernel(const float* __rest
                                                             float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot,
                                                             const int* __restrict__ pos, const int* __restrict__ slot, const int* __restrict__ table,
                                                             int table_stride, TQ* __restrict__ q_out, TC* __restrict__ cache, long page_stride,
-                                                            int page_size, int n_heads, int n_kv, int hd, int vd) {
+                                                            int page_size, int n_heads, int n_kv, int hd, int vd,
+                                                            const float* __restrict__ q_bias, const float* __restrict__ k_bias,
+                                                            const float* __restrict__ v_bias, const float* __restrict__ v_other, long ld_other,
+                                                            const float* __restrict__ v_blend, float* __restrict__ v_keep, long ld_keep) {
     __shared__ float s[NRS_MAX_HD];
     const int t = blockIdx.x, item = blockIdx.y, lane = threadIdx.x;
     const int p = pos[t];
@@ -427,16 +435,24 @@ __global__ __launch_bounds__(64) void norm_rope_store_kernel(const float* __rest
         const int h = item - n_heads - n_kv;
         const long page = table[(size_t)slot[t] * table_stride + p / page_size];
         TC* vbase = cache + page * page_stride + (size_t)n_kv * page_size * hd + (size_t)h * vd * page_size + p % page_size;
-        for (int d = lane; d < vd; d += 64) store_f32(vbase, (size_t)d * page_size, v[(size_t)t * ldv + h * vd + d]);
+        const float blend = v_other ? v_blend[0] : 0.f;
+        for (int d = lane; d < vd; d += 64) {
+            float x = v[(size_t)t * ldv + h * vd + d];
+            if (v_bias) x += v_bias[h * vd + d];
+            if (v_keep) v_keep[(size_t)t * ld_keep + h * vd + d] = x;
+            if (v_other) x = (1.0f - blend) * x + blend * v_other[(size_t)t * ld_other + h * vd + d];
+            store_f32(vbase, (size_t)d * page_size, x);
+        }
         return;
     }
     const bool is_q = item < n_heads;
     const int h = is_q ? item : item - n_heads;
     const float* src = is_q ? q + (size_t)t * ldq + h * hd : k + (size_t)t * ldk + h * hd;
+    const float* bias = is_q ? q_bias : k_bias;
     const TW* w = is_q ? q_norm : k_norm;
     float ss = 0.f;
     for (int d = lane; d < hd; d += 64) {
-        const float x = src[d];
+        const float x = bias ? src[d] + bias[h * hd + d] : src[d];
         s[d] = x;
         ss = fmaf(x, x, ss);
     }
@@ -468,9 +484,14 @@ __global__ __launch_bounds__(64) void norm_rope_store_kernel(const float* __rest
 GI_API int gi_norm_rope_store(const float* q, const float* k, const float* v, long ldq, long ldk, long ldv, const void* q_norm, const void* k_norm,
                               int norm_dtype, float eps, const float* cos_t, const float* sin_t, int rot, const int* pos, const int* slot,
                               const int* table, int table_stride, void* q_out, int q_dtype, void* cache, int cache_dtype, long page_stride,
-                              int page_size, int n_rows, int n_heads, int n_kv, int hd, int vd, hipStream_t stream) {
+                              int page_size, int n_rows, int n_heads, int n_kv, int hd, int vd, const float* q_bias, const float* k_bias,
+                              const float* v_bias, const float* v_other, long ld_other, const float* v_blend, float* v_keep, long ld_keep,
+                              hipStream_t stream) {
     GI_REQUIRE(n_rows > 0 && n_heads > 0 && n_kv > 0 && hd > 0 && hd <= NRS_MAX_HD && vd > 0, "norm_rope_store: bad sizes (rows %d heads %d kv %d hd %d vd %d)",
                n_rows, n_heads, n_kv, hd, vd);
+    GI_REQUIRE((v_other == nullptr || (v_blend != nullptr && ld_other >= (long)n_kv * vd)) && (v_keep == nullptr || ld_keep >= (long)n_kv * vd) &&
+               ((v_other == nullptr && v_keep == nullptr && v_bias == nullptr && k_bias == nullptr) || k != nullptr),
+               "norm_rope_store: blended, kept or biased values need values of this layer's own, the blend's weight and rows of n_kv*vd numbers");
     GI_REQUIRE((cos_t == nullptr) == (sin_t == nullptr) && rot >= 0 && rot % 2 == 0 && rot <= hd, "norm_rope_store: cos and sin go together, and the rotated channels are an even number within the head");
     GI_REQUIRE(k == nullptr || (v != nullptr && cache != nullptr && table != nullptr && page_size > 0 && page_stride >= (long)n_kv * page_size * (hd + vd)),
                "norm_rope_store: a cache write needs v, a cache, a table and a page stride of at least n_kv*page_size*(hd+vd)");
@@ -478,7 +499,8 @@ GI_API int gi_norm_rope_store(const float* q, const float* k, const float* v, lo
     dim3 grid(n_rows, n_heads + (k ? 2 * n_kv : 0));
 #define LAUNCH(TQ, TC, TW)                                                                                                                    \
     norm_rope_store_kernel<TQ, TC, TW><<<grid, 64, 0, stream>>>(q, k, v, ldq, ldk, ldv, (const TW*)q_norm, (const TW*)k_norm, eps, cos_t, sin_t, rot, pos, \
-                                                                slot, table, table_stride, (TQ*)q_out, (TC*)cache, page_stride, page_size, n_heads, n_kv, hd, vd)
+                                                                slot, table, table_stride, (TQ*)q_out, (TC*)cache, page_stride, page_size, n_heads, n_kv, hd, vd, \
+                                                                q_bias, k_bias, v_bias, v_other, ld_other, v_blend, v_keep, ld_keep)
     if (q_dtype == GI_F32 && cache_dtype == GI_F32 && norm_dtype == GI_F32) LAUNCH(float, float, float);
     else if (q_dtype == GI_BF16 && cache_dtype == GI_BF16 && norm_dtype == GI_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);
     else if (q_dtype == GI_BF16 && cache_dtype == GI_BF16 && norm_dtype == GI_F32) LAUNCH(bf16_t, bf16_t, float);
@@ -509,6 +531,34 @@ GI_API int gi_act_mul(const float* gate_up, void* h, int h_dtype, int n_rows, in
     else if (h_dtype == GI_BF16) act_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>(gate_up, (bf16_t*)h, inter, n, act);
     else return gi_fail("act_mul: unknown dtype %d", h_dtype);
     GI_CHECK_LAUNCH("act_mul");
+    return 0;
+}
+
+// ------------------------------------------------------------------------- feed-forward without a gate
+// h[t, i] = act(x[t, i]) for the two-parameter activation "xielu": with a = softplus(params[0]) and b = 1/2 + softplus(params[1]),
+//   z > 0:  a z^2 + z / 2          z <= 0:  b (exp(z) - 1 - z) + z / 2
+// (quadratic on the right, bounded below on the left, slope 1/2 on both sides of 0).  params: two float32 numbers on the device.
+__device__ __forceinline__ float softplus_f32(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+template <typename TO>
+__global__ void xielu_kernel(const float* __restrict__ x, long ldx, TO* __restrict__ h, long ldh, int inter, size_t n, const float* __restrict__ params) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const size_t t = i / inter, c = i % inter;
+    const float a = softplus_f32(params[0]), b = 0.5f + softplus_f32(params[1]);
+    const float z = x[t * ldx + c];
+    const float y = z > 0.f ? fmaf(a * z, z, 0.5f * z) : fmaf(b, expm1f(z) - z, 0.5f * z);
+    store_f32(h, t * ldh + c, y);
+}
+
+GI_API int gi_xielu(const float* x, long ldx, void* h, int h_dtype, long ldh, int n_rows, int inter, const float* params, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && inter > 0 && ldx >= inter && ldh >= inter && params != nullptr, "xielu: bad sizes (rows %d, columns %d) or no parameters", n_rows, inter);
+    const size_t n = (size_t)n_rows * inter;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (h_dtype == GI_F32) xielu_kernel<float><<<blocks, 256, 0, stream>>>(x, ldx, (float*)h, ldh, inter, n, params);
+    else if (h_dtype == GI_BF16) xielu_kernel<bf16_t><<<blocks, 256, 0, stream>>>(x, ldx, (bf16_t*)h, ldh, inter, n, params);
+    else return gi_fail("xielu: unknown dtype %d", h_dtype);
+    GI_CHECK_LAUNCH("xielu");
     return 0;
 }
 

@@ -21,6 +21,14 @@
 // at once, lane by token: m runs along them one after the other (an addition and a maximum each), and the exponentials it needs
 // are then taken for all 64 at once.  Every sum's order is fixed by dk alone: a request's results have the same bits however
 // its rows are cut into steps.
+//
+// The gated delta rule keeps a memory S [dk][dv] per head and, per token with decay g, step size beta, unit key k, query q:
+//     S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q
+// (what the memory holds along k is moved towards v, then read with q: the read-out sees the token's own write).  Columns of S
+// never meet here either, so a wave owns four of them, lanes as above; a token costs two sums over the key's rows instead of
+// one, the second of which waits for the first.  Before the rule, q, k and v pass a short causal convolution over the
+// request's rows (the last taps - 1 rows before a step are part of the request's state) and SiLU, and q and k are made unit
+// vectors; after it, a head's output is divided by its root mean square, as the matrix memory's.
 #include "common.h"
 
 namespace {
@@ -198,10 +206,11 @@ __global__ __launch_bounds__(64) void mlstm_scan_kernel(const float* __restrict_
 
 // y[t, h*dv + d] = w[h*dv + d] * o[t, h, d] * rsqrt(mean_d(o[t, h, :]^2) + eps) * sigmoid(g[t, h*dv + d]): one wave per (row, head).
 // With `den` [rows, heads], o is what the rows hold divided by den[t, h] (the matrix memory's sums and their divisor).
+// w_head_stride: dv where every head has weights of its own, 0 where all heads share one [dv]; gate_act 0: sigmoid(g), 1: SiLU, g sigmoid(g).
 template <typename TW, typename TO>
 __global__ __launch_bounds__(64) void head_norm_gate_kernel(const float* __restrict__ o, long ldo, const float* __restrict__ den,
                                                            const float* __restrict__ g, long ldg, const TW* __restrict__ w,
-                                                           TO* __restrict__ y, long ldy, int n_heads, int dv, float eps) {
+                                                           TO* __restrict__ y, long ldy, int n_heads, int dv, float eps, int w_head_stride, int gate_act) {
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const float* orow = o + (size_t)t * ldo + (size_t)h * dv;
     const float by = den ? den[(size_t)t * n_heads + h] : 1.0f;
@@ -213,8 +222,163 @@ __global__ __launch_bounds__(64) void head_norm_gate_kernel(const float* __restr
     const float r = 1.0f / sqrtf(wave_sum(ss) / (float)dv + eps);
     for (int d = lane; d < dv; d += 64) {
         const float v = den ? orow[d] / by : orow[d];
-        const float gate = 1.0f / (1.0f + expf(-g[(size_t)t * ldg + (size_t)h * dv + d]));
-        store_f32(y, (size_t)t * ldy + (size_t)h * dv + d, load_f32(w, (size_t)h * dv + d) * (v * r) * gate);
+        const float z = g[(size_t)t * ldg + (size_t)h * dv + d];
+        const float gate = (gate_act ? z : 1.0f) / (1.0f + expf(-z));
+        store_f32(y, (size_t)t * ldy + (size_t)h * dv + d, load_f32(w, (size_t)h * w_head_stride + d) * (v * r) * gate);
+    }
+}
+
+
+// ------------------------------------------------------------------------------------- gated delta rule
+constexpr int DELTA_MAX_TAPS = 8;
+
+__device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+// How many of the rows before row t belong to the same request's run in this step, up to `most`.
+__device__ __forceinline__ int rows_before(const int* __restrict__ slot, const int* __restrict__ pos, int t, int most) {
+    int r = 0;
+    while (r < most && t - r - 1 >= 0 && slot[t - r - 1] == slot[t] && pos[t - r - 1] == pos[t] - r - 1) ++r;
+    return r;
+}
+
+// What the rule needs of one row, one wave per (row, item).  The convolved columns of `proj` are [conv_off, conv_off + n_conv):
+// query heads [n_kv][dk], key heads [n_kv][dk], value heads [n_heads][dv], in this order; `taps` [n_conv][n_taps] float32, the
+// last tap the row's own; `tail` [slots][n_taps - 1][n_conv] the request's last rows before this step (zeros at its start).
+//   items 0 .. 2 n_kv - 1     a query or key head: convolution, SiLU, divided by sqrt(sum of squares + 1e-6); queries times q_scale
+//   items 2 n_kv .. + n_heads a value head: convolution, SiLU
+//   the last item             per head the decay exp(-exp(a_log) softplus(pre_a + dt_bias)) and the step size sigmoid(pre_b)
+// qkv: float32 [rows, n_conv] in the columns' order; gates: float32 [rows, 2 n_heads], decays then step sizes.
+__global__ __launch_bounds__(64) void delta_prepare_kernel(const float* __restrict__ proj, long ld, int conv_off, int a_off, int b_off,
+                                                          const float* __restrict__ taps, int n_taps, const float* __restrict__ tail, long tail_stride,
+                                                          const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+                                                          const int* __restrict__ slot, const int* __restrict__ pos, float* __restrict__ qkv,
+                                                          float* __restrict__ gates, int n_heads, int n_kv, int dk, int dv, float q_scale) {
+    const int t = blockIdx.x, item = blockIdx.y, lane = threadIdx.x;
+    if (item == 2 * n_kv + n_heads) {
+        for (int h = lane; h < n_heads; h += 64) {
+            const float pre_a = proj[(size_t)t * ld + a_off + h], pre_b = proj[(size_t)t * ld + b_off + h];
+            gates[(size_t)t * 2 * n_heads + h] = expf(-expf(a_log[h]) * softplus_f(pre_a + dt_bias[h]));
+            gates[(size_t)t * 2 * n_heads + n_heads + h] = 1.0f / (1.0f + expf(-pre_b));
+        }
+        return;
+    }
+    const int n_conv = 2 * n_kv * dk + n_heads * dv;
+    const bool unit = item < 2 * n_kv;
+    const int first = unit ? item * dk : 2 * n_kv * dk + (item - 2 * n_kv) * dv, width = unit ? dk : dv;
+    const int before = rows_before(slot, pos, t, n_taps - 1);
+    const float* old = tail + (size_t)slot[t] * tail_stride;
+    float ss = 0.f;
+    for (int d = lane; d < width; d += 64) {
+        const int c = first + d;
+        float y = 0.f;
+        for (int j = 0; j < n_taps; ++j) {
+            const int back = n_taps - 1 - j;                      // rows before t that tap j reads
+            const float x = back <= before ? proj[(size_t)(t - back) * ld + conv_off + c] : old[(size_t)(n_taps - 1 - (back - before)) * n_conv + c];
+            y = fmaf(taps[(size_t)c * n_taps + j], x, y);
+        }
+        y = y / (1.0f + expf(-y));
+        qkv[(size_t)t * n_conv + c] = y;                          // (read back below by the lane that wrote it)
+        ss = fmaf(y, y, ss);
+    }
+    if (!unit) return;
+    const float r = (item < n_kv ? q_scale : 1.0f) / sqrtf(wave_sum(ss) + 1e-6f);
+    for (int d = lane; d < width; d += 64) qkv[(size_t)t * n_conv + first + d] *= r;
+}
+
+// After a step's rows the request's tail is its last n_taps - 1 inputs: of this step's rows, and of the old tail where the step
+// brought fewer.  One workgroup per request of the step; a thread reads all it needs of a channel before it writes.
+__global__ __launch_bounds__(256) void delta_tail_kernel(const float* __restrict__ proj, long ld, int conv_off, int n_conv, int n_taps,
+                                                        const int* __restrict__ seg_start, const int* __restrict__ seg_len,
+                                                        const int* __restrict__ slot, float* __restrict__ tail, long tail_stride) {
+    const int n = seg_len[blockIdx.x];
+    if (n <= 0) return;
+    const int t0 = seg_start[blockIdx.x], keep = n_taps - 1;
+    float* mine = tail + (size_t)slot[t0] * tail_stride;
+    for (int c = threadIdx.x; c < n_conv; c += 256) {
+        float held[DELTA_MAX_TAPS];
+#pragma unroll
+        for (int s = 0; s < DELTA_MAX_TAPS; ++s) {
+            if (s >= keep) break;
+            const int e = n - keep + s;                           // row of the step, or (negative) place before it
+            held[s] = e >= 0 ? proj[(size_t)(t0 + e) * ld + conv_off + c] : mine[(size_t)(keep + e) * n_conv + c];
+        }
+#pragma unroll
+        for (int s = 0; s < DELTA_MAX_TAPS; ++s) {
+            if (s >= keep) break;
+            mine[(size_t)s * n_conv + c] = held[s];
+        }
+    }
+}
+
+// The rule itself: one wave per (request of the step, head, four columns of S).  lane = column * 16 + group of rows; a lane keeps
+// the rows 16 apart of its column.  State of a request slot: [head][tile]{[dk][4]}.  Key and query of a block of tokens wait in
+// LDS; every sum over the key's rows is the lanes' own shares in a fixed order, then the 16 groups by lane moves.
+template <int ROWS>
+__global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict__ qkv, long ld, const float* __restrict__ gates,
+                                                       const int* __restrict__ seg_start, const int* __restrict__ seg_len,
+                                                       const int* __restrict__ row_slot, float* __restrict__ state, long state_stride,
+                                                       float* __restrict__ out, long ldo, int n_heads, int n_kv, int dk, int dv) {
+    constexpr int C = 4, RG = 16, KQ = RG * ROWS;
+    constexpr int TB = (2048 / KQ) < 16 ? (2048 / KQ) : 16;      // tokens staged at a time
+    static_assert(TB >= 4, "a block of at least four tokens fits");
+    __shared__ float2 kq_s[TB][KQ];
+    __shared__ float v_s[TB][C];
+    __shared__ float2 gb_s[TB];
+    const int seg = blockIdx.x, h = blockIdx.y, vt = blockIdx.z, n_tiles = gridDim.z;
+    const int lane = threadIdx.x, c = lane / RG, rg = lane % RG;
+    const int n = seg_len[seg];
+    if (n <= 0) return;
+    const int t0 = seg_start[seg];
+    const int col = vt * C + c, kvh = h / (n_heads / n_kv);
+    const bool live = col < dv;
+    float* st = state + (size_t)row_slot[t0] * state_stride + ((size_t)h * n_tiles + vt) * ((size_t)dk * C);
+    const int q_at = kvh * dk, k_at = (n_kv + kvh) * dk, v_at = 2 * n_kv * dk + h * dv;
+
+    float S[ROWS];
+#pragma unroll
+    for (int rr = 0; rr < ROWS; ++rr) {
+        const int i = rr * RG + rg;
+        S[rr] = i < dk ? st[(size_t)i * C + c] : 0.f;
+    }
+    for (int b0 = 0; b0 < n; b0 += TB) {
+        const int here = min(TB, n - b0);
+        __syncthreads();                                          // the block before has been read
+        for (int idx = lane; idx < here * KQ; idx += 64) {
+            const int u = idx / KQ, i = idx % KQ;
+            const float* row = qkv + (size_t)(t0 + b0 + u) * ld;
+            kq_s[u][i] = i < dk ? float2{row[k_at + i], row[q_at + i]} : float2{0.f, 0.f};
+        }
+        if (lane < here * C) {
+            const int u = lane / C, cc = vt * C + lane % C;
+            v_s[u][lane % C] = cc < dv ? qkv[(size_t)(t0 + b0 + u) * ld + v_at + cc] : 0.f;
+        }
+        if (lane < here) {
+            const float* g = gates + (size_t)(t0 + b0 + lane) * 2 * n_heads;
+            gb_s[lane] = float2{g[h], g[n_heads + h]};
+        }
+        __syncthreads();
+        for (int u = 0; u < here; ++u) {
+            const float2 gb = gb_s[u];
+            float held = 0.f;
+#pragma unroll
+            for (int rr = 0; rr < ROWS; ++rr) held = fmaf(S[rr], kq_s[u][rr * RG + rg].x, held);
+            held = gb.x * group_sum<RG>(held);                    // what the decayed memory holds along the key
+            const float w = gb.y * (v_s[u][c] - held);
+            float acc = 0.f;
+#pragma unroll
+            for (int rr = 0; rr < ROWS; ++rr) {
+                const float2 kq = kq_s[u][rr * RG + rg];
+                S[rr] = fmaf(gb.x, S[rr], kq.x * w);
+                acc = fmaf(S[rr], kq.y, acc);
+            }
+            acc = group_sum<RG>(acc);
+            if (rg == 0 && live) out[(size_t)(t0 + b0 + u) * ldo + h * dv + col] = acc;
+        }
+    }
+#pragma unroll
+    for (int rr = 0; rr < ROWS; ++rr) {
+        const int i = rr * RG + rg;
+        if (i < dk) st[(size_t)i * C + c] = S[rr];
     }
 }
 
@@ -254,11 +418,68 @@ GI_API int gi_mlstm_scan(const float* proj, long ld, int q_off, int k_off, int v
     return 0;
 }
 
+// Floats of one request slot's state of the gated delta rule: the memories, per head and tile of four value channels [dk][4],
+// then the convolutions' tail [n_taps - 1][2 n_kv dk + n_heads dv].
+GI_API long gi_delta_memory_floats(int n_heads, int dk, int dv) { return (long)n_heads * ((dv + 3) / 4) * ((long)dk * 4); }
+GI_API long gi_delta_state_floats(int n_heads, int n_kv, int dk, int dv, int n_taps) {
+    return gi_delta_memory_floats(n_heads, dk, dv) + (long)(n_taps - 1) * (2L * n_kv * dk + (long)n_heads * dv);
+}
+GI_API int gi_delta_max_key_dim() { return 512; }
+GI_API int gi_delta_max_taps() { return DELTA_MAX_TAPS; }
+
+// proj: float32 [n_rows, ld]; see delta_prepare_kernel.  state: [slots, state_stride], a slot's memories then its tail.
+GI_API int gi_delta_prepare(const float* proj, long ld, int conv_off, int a_off, int b_off, const float* taps, int n_taps, const float* a_log,
+                            const float* dt_bias, const int* slot, const int* pos, float* state, long state_stride, float* qkv, float* gates,
+                            int n_rows, int n_heads, int n_kv, int dk, int dv, float q_scale, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0 && dk > 0 && dv > 0, "delta_prepare: bad sizes (rows %d, heads %d, kv heads %d, dk %d, dv %d)",
+               n_rows, n_heads, n_kv, dk, dv);
+    GI_REQUIRE(n_taps >= 1 && n_taps <= DELTA_MAX_TAPS, "delta_prepare: %d taps, 1 to %d are served", n_taps, DELTA_MAX_TAPS);
+    const long n_conv = 2L * n_kv * dk + (long)n_heads * dv;
+    GI_REQUIRE(conv_off >= 0 && a_off >= 0 && b_off >= 0 && ld >= conv_off + n_conv && ld >= a_off + n_heads && ld >= b_off + n_heads,
+               "delta_prepare: the columns named lie outside the rows");
+    GI_REQUIRE(state_stride >= gi_delta_state_floats(n_heads, n_kv, dk, dv, n_taps) && 2 * n_kv + n_heads + 1 <= 65535, "delta_prepare: state stride %ld too small, or too many heads", state_stride);
+    dim3 grid(n_rows, 2 * n_kv + n_heads + 1);
+    delta_prepare_kernel<<<grid, 64, 0, stream>>>(proj, ld, conv_off, a_off, b_off, taps, n_taps, state + gi_delta_memory_floats(n_heads, dk, dv), state_stride,
+                                                  a_log, dt_bias, slot, pos, qkv, gates, n_heads, n_kv, dk, dv, q_scale);
+    GI_CHECK_LAUNCH("delta_prepare");
+    return 0;
+}
+
+GI_API int gi_delta_tail(const float* proj, long ld, int conv_off, int n_taps, const int* seg_start, const int* seg_len, int n_segs, const int* slot,
+                         float* state, long state_stride, int n_heads, int n_kv, int dk, int dv, hipStream_t stream) {
+    GI_REQUIRE(n_segs > 0 && n_taps >= 1 && n_taps <= DELTA_MAX_TAPS, "delta_tail: %d runs, %d taps", n_segs, n_taps);
+    const long n_conv = 2L * n_kv * dk + (long)n_heads * dv;
+    GI_REQUIRE(conv_off >= 0 && ld >= conv_off + n_conv && state_stride >= gi_delta_state_floats(n_heads, n_kv, dk, dv, n_taps), "delta_tail: columns outside the rows, or state stride too small");
+    if (n_taps == 1) return 0;
+    delta_tail_kernel<<<n_segs, 256, 0, stream>>>(proj, ld, conv_off, (int)n_conv, n_taps, seg_start, seg_len, slot, state + gi_delta_memory_floats(n_heads, dk, dv), state_stride);
+    GI_CHECK_LAUNCH("delta_tail");
+    return 0;
+}
+
+// qkv: float32 [n_rows, ld], a row's unit queries [n_kv][dk], unit keys [n_kv][dk], values [n_heads][dv]; gates: float32 [n_rows, 2 n_heads];
+// out: float32 [n_rows, ldo] gets the heads' read-outs [n_heads][dv].
+GI_API int gi_delta_scan(const float* qkv, long ld, const float* gates, const int* seg_start, const int* seg_len, int n_segs, const int* row_slot,
+                         float* state, long state_stride, float* out, long ldo, int n_heads, int n_kv, int dk, int dv, hipStream_t stream) {
+    GI_REQUIRE(n_segs > 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0 && dk > 0 && dk <= 512 && dv > 0, "delta_scan: bad sizes (runs %d, heads %d, kv heads %d, dk %d, dv %d; dk at most 512)",
+               n_segs, n_heads, n_kv, dk, dv);
+    GI_REQUIRE(ld >= 2L * n_kv * dk + (long)n_heads * dv && ldo >= (long)n_heads * dv && state_stride >= gi_delta_memory_floats(n_heads, dk, dv), "delta_scan: row or state strides too small");
+    const int tiles = (dv + 3) / 4;
+    GI_REQUIRE(n_heads <= 65535 && tiles <= 65535, "delta_scan: too many heads or value channels");
+    dim3 grid(n_segs, n_heads, tiles);
+#define GO(R) delta_scan_kernel<R><<<grid, 64, 0, stream>>>(qkv, ld, gates, seg_start, seg_len, row_slot, state, state_stride, out, ldo, n_heads, n_kv, dk, dv)
+    if (dk <= 32) GO(2); else if (dk <= 64) GO(4); else if (dk <= 128) GO(8); else if (dk <= 256) GO(16); else GO(32);
+#undef GO
+    GI_CHECK_LAUNCH("delta_scan");
+    return 0;
+}
+
 GI_API int gi_head_norm_gate(const float* o, long ldo, const float* den, const float* g, long ldg, const void* w, int w_dtype, void* y, int y_dtype, long ldy, int n_rows,
-                             int n_heads, int dv, float eps, hipStream_t stream) {
+                             int n_heads, int dv, float eps, int shared_weight, int gate_act, hipStream_t stream) {
     GI_REQUIRE(n_rows > 0 && n_heads > 0 && n_heads <= 65535 && dv > 0, "head_norm_gate: bad sizes (rows %d, heads %d, dv %d)", n_rows, n_heads, dv);
+    GI_REQUIRE(gate_act == 0 || gate_act == 1, "head_norm_gate: the gate is a sigmoid (0) or SiLU (1)");
     dim3 grid(n_rows, n_heads);
-#define GO(TW, TO) head_norm_gate_kernel<TW, TO><<<grid, 64, 0, stream>>>(o, ldo, den, g, ldg, (const TW*)w, (TO*)y, ldy, n_heads, dv, eps)
+    const int w_head_stride = shared_weight ? 0 : dv;
+#define GO(TW, TO) head_norm_gate_kernel<TW, TO><<<grid, 64, 0, stream>>>(o, ldo, den, g, ldg, (const TW*)w, (TO*)y, ldy, n_heads, dv, eps, w_head_stride, gate_act)
     if (w_dtype == GI_F32 && y_dtype == GI_F32) GO(float, float);
     else if (w_dtype == GI_F32 && y_dtype == GI_BF16) GO(float, bf16_t);
     else if (w_dtype == GI_BF16 && y_dtype == GI_BF16) GO(bf16_t, bf16_t);

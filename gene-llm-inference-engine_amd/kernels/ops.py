@@ -26,7 +26,7 @@ _SIGNATURES = {
     "gi_embed": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "gi_embed_handing": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
     "gi_rmsnorm": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_long, c_long, c_void_p],
-    "gi_rope_cos_sin": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "gi_rope_cos_sin": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p],
     "gi_rope_store": [c_void_p, c_void_p, c_void_p, c_long, c_long, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                       c_int, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gi_silu_mul": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
@@ -35,16 +35,25 @@ _SIGNATURES = {
     "gi_softcap_rows": [c_void_p, c_int, c_int, c_long, c_float, c_void_p],
     "gi_gemm_exact": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p],
     "gi_attention_exact": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int,
-                           c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_long, c_void_p],
+                           c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_long, c_int, c_void_p],
     "gi_rmsnorm_add": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_long, c_long, c_void_p],
     "gi_rmsnorm_add_norm": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_long, c_long, c_long, c_void_p],
     "gi_norm_rope_store": [c_void_p, c_void_p, c_void_p, c_long, c_long, c_long, c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int,
-                           c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                           c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int,
+                           c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_long, c_void_p],
+    "gi_xielu": [c_void_p, c_long, c_void_p, c_int, c_long, c_int, c_int, c_void_p, c_void_p],
+    "gi_delta_prepare": [c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p,
+                         c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+    "gi_delta_tail": [c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p],
+    "gi_delta_scan": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_long, c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p],
+    "gi_latent_prepare": [c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                          c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_int, c_int, c_void_p],
+    "gi_latent_queries": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gi_act_mul": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "gi_segments": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p],
     "gi_mlstm_scan": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_int, c_void_p,
                       c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_void_p],
-    "gi_head_norm_gate": [c_void_p, c_long, c_void_p, c_void_p, c_long, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_float, c_void_p],
+    "gi_head_norm_gate": [c_void_p, c_long, c_void_p, c_void_p, c_long, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
     "gi_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long, c_void_p],
     "gi_attention_prompt_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
                                  c_float, c_int, c_void_p, c_void_p, c_int, c_void_p, c_long, c_int, c_void_p, c_void_p, c_long, c_void_p],
@@ -282,8 +291,8 @@ def rmsnorm(x, weight, eps, out, rows=None):
     return out
 
 
-def rope_cos_sin(positions, inv_freq, cos_out, sin_out):
-    """cos/sin of positions[t] * inv_freq[k] with 64-bit angles; outputs float32 [n, half]."""
+def rope_cos_sin(positions, inv_freq, cos_out, sin_out, magnitude: float = 1.0):
+    """magnitude * cos/sin of positions[t] * inv_freq[k] with 64-bit angles; outputs float32 [n, half]."""
     _dev(positions, inv_freq, cos_out, sin_out)
     n, half = cos_out.shape
     _i32(positions, "rope_cos_sin: positions", n)
@@ -292,7 +301,7 @@ def rope_cos_sin(positions, inv_freq, cos_out, sin_out):
     for t in (cos_out, sin_out):
         if not (t.dtype == torch.float32 and t.is_contiguous() and t.shape == (n, half)):
             raise KernelError("rope_cos_sin: outputs must be float32 [n, half]")
-    _call("gi_rope_cos_sin", positions.data_ptr(), inv_freq.data_ptr(), cos_out.data_ptr(), sin_out.data_ptr(), n, half, _stream())
+    _call("gi_rope_cos_sin", positions.data_ptr(), inv_freq.data_ptr(), cos_out.data_ptr(), sin_out.data_ptr(), n, half, float(magnitude), _stream())
 
 
 def _check_cache(cache, table, page_size, n_kv, hd, what):
@@ -420,11 +429,12 @@ def _check_paged(cache, table, what):
 
 
 def attention_exact(q, cache, out, positions, slots, table, n_heads, n_kv, hd, window=None, scale=None, *, page_size=None, value_dim=None,
-                    chunk=None, sinks=None, gate=None):
+                    chunk=None, sinks=None, gate=None, values_in_keys=False):
     """Each row attends over its request's cached keys up to its own position, no further back than `window` positions and not
     beyond the start of its own chunk of `chunk` positions.  value_dim: channels of a value head (hd if not given); sinks:
     float32 [heads], a score per head that joins the softmax's denominator only; gate: float32 [n, >= heads] (unit inner
-    stride), head h's output is multiplied by sigmoid(gate[t, h])."""
+    stride), head h's output is multiplied by sigmoid(gate[t, h]).  values_in_keys: the pages hold keys only, and a position's value is
+    the first value_dim channels of its key."""
     _dev(q, cache, out, positions, slots, table, sinks, gate)
     n = q.shape[0]
     vd = int(value_dim or hd)
@@ -444,7 +454,7 @@ def attention_exact(q, cache, out, positions, slots, table, n_heads, n_kv, hd, w
     _call("gi_attention_exact", q.data_ptr(), _code(q, "attention: q"), cache.data_ptr(), _code(cache, "attention: cache"), out.data_ptr(),
           _code(out, "attention: out"), positions.data_ptr(), slots.data_ptr(), table.data_ptr(), table.stride(0), cache.stride(0),
           page_size, n, n_heads, n_kv, hd, vd, int(window or 0), int(chunk or 0), float(scale if scale is not None else hd ** -0.5),
-          _ptr(sinks), _ptr(gate), gate.stride(0) if gate is not None else 0, _stream())
+          _ptr(sinks), _ptr(gate), gate.stride(0) if gate is not None else 0, 1 if values_in_keys else 0, _stream())
     return out
 
 
@@ -474,11 +484,29 @@ def rmsnorm_add_norm(y, weight, eps, x, next_weight, next_eps, out):
     return out
 
 
-def norm_rope_store(q, k, v, q_norm, k_norm, eps, cos, sin, rotary_dim, positions, slots, table, q_out, cache, page_size, n_heads, n_kv, hd, vd):
+def norm_rope_store(q, k, v, q_norm, k_norm, eps, cos, sin, rotary_dim, positions, slots, table, q_out, cache, page_size, n_heads, n_kv, hd, vd,
+                    biases=None, blend=None, keep=None):
     """The general form of `rope_store`: every query and key head is first RMS-normed with q_norm / k_norm [hd] (None: not), then
     the pairs (i, i + rotary_dim/2) of its first rotary_dim channels are turned (cos, sin float32 [n, rotary_dim/2]; None: not);
-    queries go to q_out, keys and the values (vd channels a head) into the cache's pages.  k None: the pages are another layer's."""
+    queries go to q_out, keys and the values (vd channels a head) into the cache's pages.  k None: the pages are another layer's.
+    biases = (q_bias, k_bias, v_bias): float32 vectors added to the products first (each may be None).  blend = (other, weight):
+    the values that go into the pages are (1 - weight) v + weight other, other float32 [n, kv_heads*vd] (another layer's values of
+    the same rows), weight one float32 number on the device.  keep: float32 [n, kv_heads*vd], gets this layer's values (with
+    their bias, before any blending)."""
     _dev(q, k, v, q_norm, k_norm, cos, sin, positions, slots, table, q_out, cache)
+    q_bias, k_bias, v_bias = biases if biases is not None else (None, None, None)
+    other, weight = blend if blend is not None else (None, None)
+    _dev(q_bias, k_bias, v_bias, other, weight, keep)
+    for b, width, name in ((q_bias, n_heads * hd, "q"), (k_bias, n_kv * hd, "k"), (v_bias, n_kv * vd, "v")):
+        if b is not None and not (b.dtype == torch.float32 and b.is_contiguous() and b.numel() == width):
+            raise KernelError(f"norm_rope_store: the {name} bias must be float32 [{width}]")
+    for rows, name in ((other, "blended"), (keep, "kept")):
+        if rows is not None and not (k is not None and rows.dtype == torch.float32 and rows.dim() == 2 and rows.shape == (q.shape[0], n_kv * vd) and rows.stride(1) == 1):
+            raise KernelError(f"norm_rope_store: the {name} values must be float32 [n, kv_heads*vd], beside values of the layer's own")
+    if other is not None and not (weight is not None and weight.dtype == torch.float32 and weight.numel() == 1):
+        raise KernelError("norm_rope_store: the blend's weight must be one float32 number on the device")
+    if k is None and (k_bias is not None or v_bias is not None):
+        raise KernelError("norm_rope_store: biases on keys and values need keys and values")
     n = q.shape[0]
     if not (q.dtype == torch.float32 and q.shape[1] == n_heads * hd and q.stride(1) == 1 and q_out.shape == (n, n_heads * hd) and q_out.is_contiguous()):
         raise KernelError("norm_rope_store: q must be float32 [n, heads*hd] and q_out [n, heads*hd], contiguous")
@@ -506,7 +534,21 @@ def norm_rope_store(q, k, v, q_norm, k_norm, eps, cos, sin, rotary_dim, position
           _ptr(q_norm), _ptr(k_norm), norm_code if norm_code is not None else F32, float(eps), _ptr(cos), _ptr(sin), 2 * half, positions.data_ptr(),
           slots.data_ptr(), _ptr(table) if k is not None else None, table.stride(0) if k is not None else 0, q_out.data_ptr(),
           _code(q_out, "norm_rope_store: q_out"), _ptr(cache) if k is not None else None, cache_code, cache.stride(0) if k is not None else 0,
-          int(page_size), n, n_heads, n_kv, hd, vd, _stream())
+          int(page_size), n, n_heads, n_kv, hd, vd, _ptr(q_bias), _ptr(k_bias), _ptr(v_bias), _ptr(other), other.stride(0) if other is not None else 0,
+          _ptr(weight), _ptr(keep), keep.stride(0) if keep is not None else 0, _stream())
+
+
+def xielu(x, out, params):
+    """out[t, i] = a z^2 + z/2 for z = x[t, i] > 0, else b (exp(z) - 1 - z) + z/2, with a = softplus(params[0]), b = 1/2 + softplus(params[1]);
+    x float32 [n, columns] and out [n, columns] (unit inner stride), params two float32 numbers on the device."""
+    _dev(x, out, params)
+    n, inter = out.shape
+    if not (x.dtype == torch.float32 and x.shape == (n, inter) and x.stride(1) == 1 and out.stride(1) == 1):
+        raise KernelError("xielu: x must be float32 [n, columns] and out [n, columns], with unit inner stride")
+    if not (params.dtype == torch.float32 and params.is_contiguous() and params.numel() == 2):
+        raise KernelError("xielu: the two parameters must be float32 [2]")
+    _call("gi_xielu", x.data_ptr(), x.stride(0), out.data_ptr(), _code(out, "xielu: out"), out.stride(0), n, inter, params.data_ptr(), _stream())
+    return out
 
 
 ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
@@ -582,10 +624,14 @@ def mlstm_scan(proj, offsets, i_bias, f_bias, cap, q_scale, seg_start, seg_len, 
     return out
 
 
-def head_norm_gate(o, gate, weight, eps, out, n_heads, dv, den=None):
+GATES = {"sigmoid": 0, "silu": 1}
+
+
+def head_norm_gate(o, gate, weight, eps, out, n_heads, dv, den=None, gate_activation="sigmoid"):
     """out[t, h*dv + d] = weight[h*dv + d] * o[t, h, d] * rsqrt(mean over d of o[t, h, :]^2 + eps) * sigmoid(gate[t, h*dv + d]);
     o and gate float32 [n, heads*dv] (unit inner stride: columns of a wider product are fine).  den: float32 [n, heads]; o is
-    then what the rows hold divided by den[t, h]."""
+    then what the rows hold divided by den[t, h].  weight may be [dv] instead: one for all heads.  gate_activation "silu": the
+    last factor is gate * sigmoid(gate)."""
     _dev(o, gate, weight, out, den)
     n = o.shape[0]
     if den is not None and not (den.dtype == torch.float32 and den.shape == (n, n_heads) and den.is_contiguous()):
@@ -593,11 +639,144 @@ def head_norm_gate(o, gate, weight, eps, out, n_heads, dv, den=None):
     for t, name in ((o, "o"), (gate, "gate")):
         if not (t.dtype == torch.float32 and t.shape == (n, n_heads * dv) and t.stride(1) == 1):
             raise KernelError(f"head_norm_gate: {name} must be float32 [n, heads*dv]")
-    if not (weight.numel() == n_heads * dv and weight.is_contiguous() and out.shape == (n, n_heads * dv) and out.stride(1) == 1):
-        raise KernelError("head_norm_gate: weight must be [heads*dv] and out [n, heads*dv]")
+    shared = weight.numel() == dv and n_heads > 1
+    if not (weight.numel() in (n_heads * dv, dv) and weight.is_contiguous() and out.shape == (n, n_heads * dv) and out.stride(1) == 1):
+        raise KernelError("head_norm_gate: weight must be [heads*dv] or [dv], and out [n, heads*dv]")
+    if gate_activation not in GATES:
+        raise KernelError(f"head_norm_gate: unknown gate {gate_activation!r}; known: {', '.join(GATES)}")
     _call("gi_head_norm_gate", o.data_ptr(), o.stride(0), _ptr(den), gate.data_ptr(), gate.stride(0), weight.data_ptr(), _code(weight, "head_norm_gate: weight"),
-          out.data_ptr(), _code(out, "head_norm_gate: out"), out.stride(0), n, n_heads, dv, float(eps), _stream())
+          out.data_ptr(), _code(out, "head_norm_gate: out"), out.stride(0), n, n_heads, dv, float(eps), 1 if shared else 0, GATES[gate_activation], _stream())
     return out
+
+
+# ------------------------------------------------------------------------------------------------ the gated delta rule
+DELTA_MAX_KEY_DIM, DELTA_MAX_TAPS = 512, 8
+
+
+def delta_memory_floats(n_heads, dk, dv) -> int:
+    """32-bit numbers of one request's memories of the gated delta rule, as `delta_scan` lays them out: per head and tile of four
+    value channels, [dk][4]."""
+    return n_heads * (-(-dv // 4)) * dk * 4
+
+
+def delta_state_floats(n_heads, n_kv, dk, dv, n_taps) -> int:
+    """... and of its whole state: the memories, then the convolutions' last n_taps - 1 inputs [n_taps - 1][2 n_kv dk + n_heads dv]
+    (needs no library, so that a cache can be planned without one)."""
+    return delta_memory_floats(n_heads, dk, dv) + (n_taps - 1) * (2 * n_kv * dk + n_heads * dv)
+
+
+def _delta_checks(what, proj, state, n_heads, n_kv, dk, dv, n_taps):
+    if not (proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1):
+        raise KernelError(f"{what}: the projections must be float32 [n, columns] with unit inner stride")
+    if not (state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1 and state.shape[1] >= delta_state_floats(n_heads, n_kv, dk, dv, n_taps)):
+        raise KernelError(f"{what}: state must be float32 [slots, delta_state_floats]")
+    if not (0 < dk <= DELTA_MAX_KEY_DIM and 1 <= n_taps <= DELTA_MAX_TAPS and n_heads % n_kv == 0):
+        raise KernelError(f"{what}: keys of 1 to {DELTA_MAX_KEY_DIM} channels, 1 to {DELTA_MAX_TAPS} taps and heads in whole groups are served")
+
+
+def delta_prepare(proj, conv_off, a_off, b_off, taps, a_log, dt_bias, ctx_slots, ctx_positions, state, qkv, gates, n_heads, n_kv, dk, dv, q_scale):
+    """What the gated delta rule needs of every row (csrc/recurrent.hip: delta_prepare_kernel): the columns [conv_off, conv_off +
+    2 n_kv dk + n_heads dv) of proj (queries, keys, values) through their short convolutions (taps float32 [channels, n_taps]; a
+    request's rows before this step come from its state) and SiLU, queries and keys made unit vectors per head (queries times
+    q_scale), into qkv float32 [n, channels]; and gates float32 [n, 2 heads]: the decays exp(-exp(a_log) softplus(proj[a_off + h] +
+    dt_bias)), then the step sizes sigmoid(proj[b_off + h])."""
+    _dev(proj, taps, a_log, dt_bias, ctx_slots, ctx_positions, state, qkv, gates)
+    n, n_conv = proj.shape[0], 2 * n_kv * dk + n_heads * dv
+    n_taps = taps.shape[1]
+    _delta_checks("delta_prepare", proj, state, n_heads, n_kv, dk, dv, n_taps)
+    if not (taps.dtype == torch.float32 and taps.shape == (n_conv, n_taps) and taps.is_contiguous()):
+        raise KernelError("delta_prepare: taps must be float32 [2 kv_heads dk + heads dv, n_taps]")
+    for t, name in ((a_log, "a_log"), (dt_bias, "dt_bias")):
+        if not (t.dtype == torch.float32 and t.is_contiguous() and t.numel() == n_heads):
+            raise KernelError(f"delta_prepare: {name} must be float32 [heads]")
+    if not (qkv.dtype == torch.float32 and qkv.shape == (n, n_conv) and qkv.is_contiguous() and gates.dtype == torch.float32 and gates.shape == (n, 2 * n_heads) and gates.is_contiguous()):
+        raise KernelError("delta_prepare: qkv must be float32 [n, channels] and gates float32 [n, 2 heads], contiguous")
+    if min(conv_off, a_off, b_off) < 0 or max(conv_off + n_conv, a_off + n_heads, b_off + n_heads) > proj.shape[1]:
+        raise KernelError("delta_prepare: the columns named lie outside proj")
+    _i32(ctx_slots, "delta_prepare: slots", n)
+    _i32(ctx_positions, "delta_prepare: positions", n)
+    _call("gi_delta_prepare", proj.data_ptr(), proj.stride(0), int(conv_off), int(a_off), int(b_off), taps.data_ptr(), n_taps, a_log.data_ptr(), dt_bias.data_ptr(),
+          ctx_slots.data_ptr(), ctx_positions.data_ptr(), state.data_ptr(), state.stride(0), qkv.data_ptr(), gates.data_ptr(), n, n_heads, n_kv, dk, dv,
+          float(q_scale), _stream())
+
+
+def delta_tail(proj, conv_off, n_taps, seg_start, seg_len, row_slot, state, n_heads, n_kv, dk, dv):
+    """After `delta_prepare` has read them: every request's last n_taps - 1 rows of the convolved columns become its state's tail."""
+    _dev(proj, seg_start, seg_len, row_slot, state)
+    _delta_checks("delta_tail", proj, state, n_heads, n_kv, dk, dv, n_taps)
+    n_segs = seg_start.numel()
+    _i32(seg_start, "delta_tail: seg_start", n_segs)
+    _i32(seg_len, "delta_tail: seg_len", n_segs)
+    _i32(row_slot, "delta_tail: slots", proj.shape[0])
+    if conv_off < 0 or conv_off + 2 * n_kv * dk + n_heads * dv > proj.shape[1]:
+        raise KernelError("delta_tail: the columns named lie outside proj")
+    _call("gi_delta_tail", proj.data_ptr(), proj.stride(0), int(conv_off), int(n_taps), seg_start.data_ptr(), seg_len.data_ptr(), n_segs, row_slot.data_ptr(),
+          state.data_ptr(), state.stride(0), n_heads, n_kv, dk, dv, _stream())
+
+
+def delta_scan(qkv, gates, seg_start, seg_len, row_slot, state, out, n_heads, n_kv, dk, dv):
+    """The gated delta rule over every request's rows of the step, in order (csrc/recurrent.hip states it): qkv and gates as
+    `delta_prepare` leaves them, out float32 [n, heads*dv] gets the read-outs S^T q; the memories come from the request's state
+    slot and go back into it."""
+    _dev(qkv, gates, seg_start, seg_len, row_slot, state, out)
+    n = qkv.shape[0]
+    if not (qkv.dtype == torch.float32 and qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] >= 2 * n_kv * dk + n_heads * dv and gates.dtype == torch.float32
+            and gates.shape == (n, 2 * n_heads) and gates.is_contiguous() and out.dtype == torch.float32 and out.shape == (n, n_heads * dv) and out.stride(1) == 1):
+        raise KernelError("delta_scan: qkv must be float32 [n, channels], gates float32 [n, 2 heads], out float32 [n, heads*dv]")
+    if not (state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1 and state.shape[1] >= delta_memory_floats(n_heads, dk, dv)):
+        raise KernelError("delta_scan: state must be float32 [slots, at least delta_memory_floats]")
+    if not (0 < dk <= DELTA_MAX_KEY_DIM and n_heads % n_kv == 0):
+        raise KernelError(f"delta_scan: keys of 1 to {DELTA_MAX_KEY_DIM} channels and heads in whole groups are served")
+    n_segs = seg_start.numel()
+    _i32(seg_start, "delta_scan: seg_start", n_segs)
+    _i32(seg_len, "delta_scan: seg_len", n_segs)
+    _i32(row_slot, "delta_scan: slots", n)
+    _call("gi_delta_scan", qkv.data_ptr(), qkv.stride(0), gates.data_ptr(), seg_start.data_ptr(), seg_len.data_ptr(), n_segs, row_slot.data_ptr(), state.data_ptr(),
+          state.stride(0), out.data_ptr(), out.stride(0), n_heads, n_kv, dk, dv, _stream())
+    return out
+
+
+# --------------------------------------------------------------------------------------------- attention through latents
+def latent_prepare(proj, q_rank, kv_rank, rot, q_norm, kv_norm, eps, cos, sin, positions, slots, table, cq, cache, page_size):
+    """proj float32 [n, q_rank + kv_rank + rot]: the query latent, RMS-normed with q_norm, into cq [n, q_rank]; the key/value latent,
+    RMS-normed with kv_norm, and the last rot channels turned in neighbouring pairs (cos, sin float32 [n, rot/2]), into the row's
+    place of its page, [place][kv_rank + rot]."""
+    _dev(proj, q_norm, kv_norm, cos, sin, positions, slots, table, cq, cache)
+    n = proj.shape[0]
+    if not (proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= q_rank + kv_rank + rot):
+        raise KernelError("latent_prepare: proj must be float32 [n, q_rank + kv_rank + rot]")
+    if not (q_norm.shape == (q_rank,) and kv_norm.shape == (kv_rank,) and q_norm.is_contiguous() and kv_norm.is_contiguous() and q_norm.dtype == kv_norm.dtype):
+        raise KernelError("latent_prepare: the norms' weights must be [q_rank] and [kv_rank], of one dtype")
+    if not (cq.shape == (n, q_rank) and cq.stride(1) == 1):
+        raise KernelError("latent_prepare: cq must be [n, q_rank]")
+    if rot:
+        for t in (cos, sin):
+            if not (t.dtype == torch.float32 and t.shape == (n, rot // 2) and t.is_contiguous()):
+                raise KernelError("latent_prepare: cos/sin must be float32 [n, rot/2]")
+    _check_paged(cache, table, "latent_prepare")
+    if cache.stride(0) < page_size * (kv_rank + rot):
+        raise KernelError("latent_prepare: the pages are too small for these latents")
+    _i32(positions, "latent_prepare: positions", n)
+    _i32(slots, "latent_prepare: slots", n)
+    _call("gi_latent_prepare", proj.data_ptr(), proj.stride(0), q_rank, kv_rank, rot, q_norm.data_ptr(), kv_norm.data_ptr(), _code(q_norm, "latent_prepare: norm"),
+          float(eps), _ptr(cos), _ptr(sin), positions.data_ptr(), slots.data_ptr(), table.data_ptr(), table.stride(0), cq.data_ptr(), _code(cq, "latent_prepare: cq"),
+          cq.stride(0), cache.data_ptr(), _code(cache, "latent_prepare: cache"), cache.stride(0), int(page_size), n, _stream())
+
+
+def latent_queries(q, cos, sin, plain, folded, n_heads, dim, rot, kv_rank):
+    """q float32 [n, heads*(dim + rot)]: every head's first dim channels into plain [n, heads*dim]; its last rot channels, turned in
+    neighbouring pairs, into folded [n, heads*(kv_rank + rot)] behind the head's first kv_rank places."""
+    _dev(q, cos, sin, plain, folded)
+    n = q.shape[0]
+    if not (q.dtype == torch.float32 and q.shape == (n, n_heads * (dim + rot)) and q.stride(1) == 1 and plain.shape == (n, n_heads * dim) and plain.stride(1) == 1
+            and folded.shape == (n, n_heads * (kv_rank + rot)) and folded.stride(1) == 1):
+        raise KernelError("latent_queries: q must be float32 [n, heads*(dim+rot)], plain [n, heads*dim], folded [n, heads*(kv_rank+rot)]")
+    if rot:
+        for t in (cos, sin):
+            if not (t.dtype == torch.float32 and t.shape == (n, rot // 2) and t.is_contiguous()):
+                raise KernelError("latent_queries: cos/sin must be float32 [n, rot/2]")
+    _call("gi_latent_queries", q.data_ptr(), q.stride(0), _ptr(cos), _ptr(sin), plain.data_ptr(), _code(plain, "latent_queries: plain"), plain.stride(0),
+          folded.data_ptr(), _code(folded, "latent_queries: folded"), folded.stride(0), n, n_heads, dim, rot, kv_rank, _stream())
 
 
 class AttentionPlan:
@@ -876,17 +1055,18 @@ def attention(q, cache, out, ctx, table, n_heads, n_kv, hd, window=None):
     return attention_exact(q, cache, out, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window)
 
 
-def attention_general(q, cache, out, ctx, table, n_heads, n_kv, hd, *, page_size, value_dim=None, window=None, chunk=None, scale=None, sinks=None, gate=None):
+def attention_general(q, cache, out, ctx, table, n_heads, n_kv, hd, *, page_size, value_dim=None, window=None, chunk=None, scale=None, sinks=None, gate=None,
+                      values_in_keys=False):
     """Attention of a step's rows for layers with any of: value heads of another size, a scale of their own, a mask cut into
-    chunks, sinks, a gate per head."""
+    chunks, sinks, a gate per head, values that are the first channels of the keys."""
     vd = int(value_dim or hd)
-    if (vd == hd and cache.dim() == 5 and q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
+    if (vd == hd and not values_in_keys and cache.dim() == 5 and q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
             and (gate is None or gate.dtype == torch.float32)):
         plan = _plan_of(ctx)
         if (not plan.n_tiles or attention_bf16_supports(hd, page_size, True)) and (not plan.n_decode or attention_bf16_supports(hd, page_size, False)):
             return attention_bf16(q, cache, out, plan, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window, scale, chunk=chunk, sinks=sinks, gate=gate)
     return attention_exact(q, cache, out, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window, scale, page_size=page_size,
-                           value_dim=value_dim, chunk=chunk, sinks=sinks, gate=gate)
+                           value_dim=value_dim, chunk=chunk, sinks=sinks, gate=gate, values_in_keys=values_in_keys)
 
 
 # Up to so many rows the decode kernel rotates and writes the pages itself.  It saves the rotation kernel's launch wherever the

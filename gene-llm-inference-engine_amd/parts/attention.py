@@ -115,6 +115,11 @@ class Attention(Mixer):
             self.sinks = None if s.sinks is None else tensors[s.sinks].float().contiguous()
             self.q_norm = None if s.q_norm is None else tensors[s.q_norm]
             self.k_norm = None if s.k_norm is None else tensors[s.k_norm]
+            as_f32 = lambda name: None if name is None else tensors[name].float().contiguous()
+            self.biases = (as_f32(s.q_bias), as_f32(s.k_bias), as_f32(s.v_bias))
+            self.value_blend = None if s.value_blend is None else tensors[s.value_blend].float().reshape(1).contiguous()
+            if s.value_blend is not None and s.value_family is None:
+                raise ValueError("attention: a blend of values needs the family whose first layer's values are blended in")
             if self.position is not None and not (hasattr(self.position, "partial_tables") or type(self.position).half_split_tables is not PositionEncoding.half_split_tables):
                 if self.q_norm is not None or self.k_norm is not None:
                     raise ValueError("attention: norms on query and key heads come before the rotation, which needs a position encoding that hands over its cosines and sines")
@@ -127,7 +132,8 @@ class Attention(Mixer):
 
     @staticmethod
     def _is_general(s) -> bool:
-        return (s.k_proj is None or any(v is not None for v in (s.value_dim, s.scale, s.chunk, s.sinks, s.q_norm, s.k_norm, s.head_gate))
+        return (s.k_proj is None or any(v is not None for v in (s.value_dim, s.scale, s.chunk, s.sinks, s.q_norm, s.k_norm, s.head_gate, s.q_bias,
+                                                                 s.k_bias, s.v_bias, s.value_family, s.value_blend))
                 or getattr(s.position, "kind", None) == "rotary_partial")
 
     @classmethod
@@ -145,6 +151,15 @@ class Attention(Mixer):
             needs.append(TensorNeed(spec.sinks, (spec.n_heads,)))
         if spec.head_gate is not None:
             needs.append(TensorNeed(spec.head_gate, (spec.n_heads, d)))
+        if spec.q_bias is not None:
+            needs.append(TensorNeed(spec.q_bias, (a,)))
+        if spec.k_proj is not None:
+            if spec.k_bias is not None:
+                needs.append(TensorNeed(spec.k_bias, (kv,)))
+            if spec.v_bias is not None:
+                needs.append(TensorNeed(spec.v_bias, (spec.n_kv_heads * vd,)))
+            if spec.value_blend is not None:
+                needs.append(TensorNeed(spec.value_blend, ()))
         return needs
 
     @classmethod
@@ -174,8 +189,19 @@ class Attention(Mixer):
             self.position.apply(q, k, ctx, s.n_heads, s.n_kv_heads, s.head_dim)
         cos, sin, turned = tables if tables is not None else (None, None, 0)
         q_ready = torch.empty((T, self.a_dim), dtype=cache.kv.dtype, device=ctx.device)
+        blend = keep = None
+        if s.value_family is not None and k is not None:
+            family = ("value_family", s.value_family)
+            if self.value_blend is None:          # the family's first layer: its values stay for the others
+                keep = ctx.memo[family] = torch.empty((T, s.n_kv_heads * vd), dtype=torch.float32, device=ctx.device)
+            else:
+                if family not in ctx.memo:
+                    raise RuntimeError(f"attention: no earlier layer of this pass has left the values of family {s.value_family!r}")
+                blend = (ctx.memo[family], self.value_blend)
+        biases = self.biases if k is not None else (self.biases[0], None, None)
         ops.norm_rope_store(q, k, v, self.q_norm, self.k_norm if k is not None else None, s.qk_norm_eps, cos, sin, turned, ctx.row_pos, ctx.row_slot,
-                            cache.table, q_ready, cache.kv, cache.page_size, s.n_heads, s.n_kv_heads, s.head_dim, vd)
+                            cache.table, q_ready, cache.kv, cache.page_size, s.n_heads, s.n_kv_heads, s.head_dim, vd,
+                            biases=biases if any(b is not None for b in biases) else None, blend=blend, keep=keep)
         att = torch.empty((T, s.n_heads * vd), dtype=cache.kv.dtype, device=ctx.device)
         return ops.attention_general(q_ready, cache.kv, att, ctx, cache.table, s.n_heads, s.n_kv_heads, s.head_dim, page_size=cache.page_size,
                                      value_dim=vd, window=s.window, chunk=s.chunk, scale=s.scale, sinks=self.sinks, gate=gate)

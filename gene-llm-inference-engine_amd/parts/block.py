@@ -4,6 +4,8 @@
     x += mixer(norm_1(x));  x += feed_forward(norm_2(x))
 "sandwich": a norm before and a norm after each half; the feed-forward half may be absent:
     x += post_1(mixer(norm_1(x)));  x += post_2(feed_forward(norm_2(x)))
+"parallel": one norm, read by the mixer and by the feed-forward (which may be absent):
+    h = norm_1(x);  x += mixer(h) + feed_forward(h)
 The residual stream x is float32 [T, hidden] and is changed in place."""
 from __future__ import annotations
 
@@ -165,3 +167,53 @@ class SandwichBlock:
 
 
 register_block("sandwich", SandwichBlock)
+
+
+class ParallelBlock:
+    """x += mixer(h) + feed_forward(h) with h = norm_1(x): both halves read the same normed rows, which are made once, and each
+    adds its result onto x (the two sums reach x one after the other; neither half reads x)."""
+
+    def __init__(self, spec, tensors, dtype, device):
+        self.spec = spec
+        if spec.feed_forward_norm is not None or spec.mixer_post_norm is not None or spec.feed_forward_post_norm is not None:
+            raise ValueError("a parallel layer has one norm, before its mixer and its feed-forward")
+        self.mixer_norm = norm_class(spec.mixer_norm)(spec.mixer_norm, tensors, dtype, device)
+        self.mixer = mixer_class(spec.mixer)(spec.mixer, tensors, dtype, device)
+        self.feed_forward = None if spec.feed_forward is None else feed_forward_class(spec.feed_forward)(spec.feed_forward, tensors, dtype, device)
+
+    def _parts(self):
+        return [self.mixer_norm, self.mixer] + ([self.feed_forward] if self.feed_forward is not None else [])
+
+    @property
+    def graph_safe(self):
+        return all(getattr(p, "graph_safe", False) for p in self._parts())
+
+    @classmethod
+    def tensor_needs(cls, spec):
+        needs = norm_class(spec.mixer_norm).tensor_needs(spec.mixer_norm) + mixer_class(spec.mixer).tensor_needs(spec.mixer)
+        if spec.feed_forward is not None:
+            needs += feed_forward_class(spec.feed_forward).tensor_needs(spec.feed_forward)
+        return needs
+
+    @classmethod
+    def cache_need(cls, spec):
+        return mixer_class(spec.mixer).cache_need(spec.mixer)
+
+    def forward(self, x, ctx, cache):
+        dtypes = {getattr(p, "in_dtype", ctx.dtype) for p in self._parts()[1:]}
+        if len(dtypes) == 1:                      # one set of normed rows serves both halves
+            h = self.mixer_norm(x, dtypes.pop())
+            rows = lambda part: h
+        else:
+            rows = lambda part: self.mixer_norm(x, getattr(part, "in_dtype", ctx.dtype))
+        h_ff = rows(self.feed_forward) if self.feed_forward is not None else None      # (made before the mixer changes x)
+        self.mixer.forward(rows(self.mixer), x, ctx, cache)
+        if ctx.trace is not None:
+            ctx.trace("attn_out", x)
+        if self.feed_forward is not None:
+            self.feed_forward.forward(h_ff, x, ctx)
+        if ctx.trace is not None:
+            ctx.trace("ffn_out", x)
+
+
+register_block("parallel", ParallelBlock)

@@ -1,0 +1,111 @@
+"""Attention through low-rank latents (`config.spec.LatentAttentionSpec` states the layer; the kernels between the products are
+`csrc/latent.hip`).
+
+What is cached per position is the normed key/value latent c [kv_rank] and one rotated key part [rotary_dim], nothing per
+head.  The up projections are folded into the two sides of the attention instead of being applied to cached rows:
+    score_j = (W_uk_h^T q_plain_h) . c_j + q_rot_h . k_rot_j        o_h = W_uv_h (sum_j p_j c_j)
+so the attention kernel sees one key/value head of kv_rank + rotary_dim channels whose first kv_rank channels are also the
+value, shared by all query heads, and every step costs the same few products whatever the context holds.
+
+Steps of a pass: one product with [W_dq; W_dkv]; one kernel that norms both latents, turns the rotated key part and writes the
+page; the product with W_uq; one kernel that parts every head's query into plain channels (rows for the folding products) and
+turned channels (written where the attention reads them); per head the folding product with W_uk_h^T; attention; per head the
+product with W_uv_h; the output product onto the residual."""
+from __future__ import annotations
+
+import torch
+
+from ..cache.needs import PagedKvNeed
+from ..kernels import ops
+from ..weights.loader import TensorNeed
+from .attention import _pad_rows
+from .base import Mixer, position_class, register_mixer
+from .linear import activation_dtype_for, linear, linear_onto
+
+
+def _head_product(a, w, out):
+    """out = a @ w.T for one head's columns of wider rows: by `linear` where the matrix-core kernels' stores find their
+    alignment in the view, by the exact kernel otherwise."""
+    if out.data_ptr() % 16 or (out.stride(0) * out.element_size()) % 16 or a.data_ptr() % 16:
+        return ops.gemm_exact(a, w, out)
+    return linear(a, w, out)
+
+
+class LatentAttention(Mixer):
+    accepts_deferred_norm = True      # its input goes into `linear` only
+    can_overwrite = True
+
+    def __init__(self, spec, tensors, dtype, device):
+        super().__init__(spec, tensors, dtype, device)
+        s = spec
+        self.key_dim = s.kv_rank + s.rotary_dim
+        if not 0 < self.key_dim <= ops.attention_max_head_size():
+            raise ValueError(f"latent attention: kv_rank + rotary_dim = {self.key_dim} is outside what the attention kernels take (up to {ops.attention_max_head_size()})")
+        if s.rotary_dim % 2:
+            raise ValueError("latent attention: the rotated channels come in pairs")
+        self.position = None
+        if s.rotary_dim:
+            if s.position is None:
+                raise ValueError("latent attention: rotated channels need a position encoding")
+            self.position = position_class(s.position)(s.position, tensors, dtype, device)
+            if not hasattr(self.position, "pair_tables") or s.position.rotary_dim != s.rotary_dim:
+                raise ValueError("latent attention: the position encoding must give angles for rotary_dim / 2 neighbouring pairs")
+        self.w_down = _pad_rows(torch.cat([tensors[s.dq_proj], tensors[s.dkv_proj]], dim=0).contiguous())
+        self.q_norm, self.kv_norm = tensors[s.dq_norm], tensors[s.dkv_norm]
+        self.w_uq = tensors[s.uq_proj]
+        # per head: W_uk_h^T [kv_rank, head_dim] (folded into the queries) and W_uv_h [value_dim, kv_rank] (applied to the attended latent)
+        self.w_uk_t = tensors[s.uk_proj].view(s.n_heads, s.head_dim, s.kv_rank).transpose(1, 2).contiguous()
+        self.w_uv = tensors[s.uv_proj].view(s.n_heads, s.value_dim, s.kv_rank)
+        self.w_o = tensors[s.o_proj]
+        self.in_dtype = activation_dtype_for(self.w_down, dtype)
+        self.cq_dtype = activation_dtype_for(self.w_uq, dtype)
+        self.plain_dtype = activation_dtype_for(self.w_uk_t, dtype)
+        self.att_dtype = activation_dtype_for(self.w_o, dtype)
+        self.graph_safe = self.position is None or bool(getattr(self.position, "graph_safe", False))
+
+    def weights_read_per_step(self):
+        return [self.w_down, self.q_norm, self.kv_norm, self.w_uq, self.w_uk_t, self.w_uv, self.w_o]
+
+    @classmethod
+    def tensor_needs(cls, spec):
+        s, d = spec, spec.hidden_size
+        return [TensorNeed(s.dq_proj, (s.q_rank, d)), TensorNeed(s.dq_norm, (s.q_rank,), "norm"), TensorNeed(s.uq_proj, (s.n_heads * (s.head_dim + s.rotary_dim), s.q_rank)),
+                TensorNeed(s.dkv_proj, (s.kv_rank + s.rotary_dim, d)), TensorNeed(s.dkv_norm, (s.kv_rank,), "norm"),
+                TensorNeed(s.uk_proj, (s.n_heads * s.head_dim, s.kv_rank)), TensorNeed(s.uv_proj, (s.n_heads * s.value_dim, s.kv_rank)),
+                TensorNeed(s.o_proj, (d, s.n_heads * s.value_dim))]
+
+    @classmethod
+    def cache_need(cls, spec):
+        return PagedKvNeed(1, spec.kv_rank + spec.rotary_dim, spec.window, spec.kv_rank, None, values_in_keys=True)
+
+    def forward(self, h, residual, ctx, cache, overwrite=False):
+        s, T, dev = self.spec, ctx.n_rows, ctx.device
+        H, kd = s.n_heads, self.key_dim
+        down = torch.empty((T, self.w_down.shape[0]), dtype=torch.float32, device=dev)
+        linear(h, self.w_down, down)
+        cos, sin = self.position.pair_tables(ctx) if self.position is not None else (None, None)
+        cq = torch.empty((T, s.q_rank), dtype=self.cq_dtype, device=dev)
+        ops.latent_prepare(down, s.q_rank, s.kv_rank, s.rotary_dim, self.q_norm, self.kv_norm, s.norm_eps, cos, sin, ctx.row_pos, ctx.row_slot,
+                           cache.table, cq, cache.kv, cache.page_size)
+        q = torch.empty((T, H * (s.head_dim + s.rotary_dim)), dtype=torch.float32, device=dev)
+        linear(cq, self.w_uq, q)
+        plain = torch.empty((T, H * s.head_dim), dtype=self.plain_dtype, device=dev)
+        folded = torch.empty((T, H * kd), dtype=cache.kv.dtype, device=dev)
+        ops.latent_queries(q, cos, sin, plain, folded, H, s.head_dim, s.rotary_dim, s.kv_rank)
+        for i in range(H):
+            _head_product(plain[:, i * s.head_dim:(i + 1) * s.head_dim], self.w_uk_t[i], folded[:, i * kd:i * kd + s.kv_rank])
+        attended = torch.empty((T, H * s.kv_rank), dtype=cache.kv.dtype, device=dev)
+        ops.attention_general(folded, cache.kv, attended, ctx, cache.table, H, 1, kd, page_size=cache.page_size, value_dim=s.kv_rank,
+                              window=s.window, scale=s.scale, values_in_keys=True)
+        if attended.dtype != activation_dtype_for(self.w_uv, self.dtype):
+            attended = attended.to(activation_dtype_for(self.w_uv, self.dtype))
+        att = torch.empty((T, H * s.value_dim), dtype=self.att_dtype, device=dev)
+        for i in range(H):
+            _head_product(attended[:, i * s.kv_rank:(i + 1) * s.kv_rank], self.w_uv[i], att[:, i * s.value_dim:(i + 1) * s.value_dim])
+        if overwrite:
+            linear(att, self.w_o, residual)
+        else:
+            linear_onto(att, self.w_o, residual)
+
+
+register_mixer("latent_attention", LatentAttention)

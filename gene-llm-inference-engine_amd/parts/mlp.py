@@ -56,3 +56,39 @@ class SwiGlu(FeedForward):
 
 
 register_feed_forward("swiglu", SwiGlu)
+
+
+class DenseMlp(FeedForward):
+    """residual += down(act(up(h))): no gate.  The activation has parameters of its own (a tensor) and runs in 32-bit on the up
+    product's rows, which it stores as the down product reads them."""
+    graph_safe = True
+    accepts_deferred_norm = True      # its input goes into `linear` only
+    can_overwrite = True
+
+    def __init__(self, spec, tensors, dtype, device):
+        super().__init__(spec, tensors, dtype, device)
+        if spec.activation != "xielu":
+            raise ValueError(f"feed-forward: unknown activation {spec.activation!r} of a dense feed-forward; known: xielu")
+        if spec.activation_params is None:
+            raise ValueError("feed-forward: the activation xielu needs its two parameters")
+        self.w_up, self.w_down = tensors[spec.up_proj], tensors[spec.down_proj]
+        self.params = tensors[spec.activation_params].float().contiguous()
+        self.in_dtype = activation_dtype_for(self.w_up, dtype)
+        self.mid_dtype = activation_dtype_for(self.w_down, dtype)
+
+    @classmethod
+    def tensor_needs(cls, spec):
+        i, d = spec.intermediate_size, spec.hidden_size
+        return [TensorNeed(spec.up_proj, (i, d)), TensorNeed(spec.down_proj, (d, i)), TensorNeed(spec.activation_params, (2,))]
+
+    def forward(self, h, residual, ctx, overwrite=False):
+        T, inter = ctx.n_rows, self.spec.intermediate_size
+        up = torch.empty((T, inter), dtype=torch.float32, device=ctx.device)
+        linear(h, self.w_up, up)
+        mid = torch.empty((T, inter), dtype=self.mid_dtype, device=ctx.device)
+        ops.xielu(up, mid, self.params)
+        linear(mid, self.w_down, residual, accumulate=not overwrite)
+        return None
+
+
+register_feed_forward("dense_mlp", DenseMlp)

@@ -28,6 +28,7 @@ class RotaryHalfSplit(PositionEncoding):
         self.half = spec.head_dim // 2
         frequencies = spec.frequencies if spec.frequencies is not None else inverse_frequencies(spec.head_dim, spec.theta)
         self.inv_freq = torch.tensor(list(frequencies), dtype=torch.float64, device=device)
+        self.magnitude = float(getattr(spec, "magnitude", 1.0))
 
     def half_split_tables(self, ctx):
         """(cos, sin), float32 [T, head_dim/2], for the rows of this step."""
@@ -35,7 +36,7 @@ class RotaryHalfSplit(PositionEncoding):
         if key not in ctx.memo:
             cos = torch.empty((ctx.n_rows, self.half), dtype=torch.float32, device=ctx.device)
             sin = torch.empty_like(cos)
-            ops.rope_cos_sin(ctx.row_pos, self.inv_freq, cos, sin)
+            ops.rope_cos_sin(ctx.row_pos, self.inv_freq, cos, sin, self.magnitude)
             ctx.memo[key] = (cos, sin)
         return ctx.memo[key]
 
@@ -50,6 +51,7 @@ class RotaryPartial(PositionEncoding):
         self.rotary_dim = spec.rotary_dim
         frequencies = spec.frequencies if spec.frequencies is not None else inverse_frequencies(spec.rotary_dim, spec.theta)
         self.inv_freq = torch.tensor(list(frequencies), dtype=torch.float64, device=device)
+        self.magnitude = float(getattr(spec, "magnitude", 1.0))
 
     def partial_tables(self, ctx):
         """(cos, sin, rotary_dim): float32 [T, rotary_dim/2] each, for the rows of this step."""
@@ -57,9 +59,32 @@ class RotaryPartial(PositionEncoding):
         if key not in ctx.memo:
             cos = torch.empty((ctx.n_rows, self.rotary_dim // 2), dtype=torch.float32, device=ctx.device)
             sin = torch.empty_like(cos)
-            ops.rope_cos_sin(ctx.row_pos, self.inv_freq, cos, sin)
+            ops.rope_cos_sin(ctx.row_pos, self.inv_freq, cos, sin, self.magnitude)
             ctx.memo[key] = (cos, sin)
         return (*ctx.memo[key], self.rotary_dim)
+
+
+class RotaryInterleaved(PositionEncoding):
+    """Angles for a rotation of neighbouring pairs (2i, 2i + 1).  It has no tables for half-split pairs and no kernel of its
+    own: a mixer whose kernels turn such pairs asks `pair_tables`."""
+    graph_safe = True
+
+    def __init__(self, spec, tensors, dtype, device):
+        super().__init__(spec, tensors, dtype, device)
+        self.rotary_dim = spec.rotary_dim
+        frequencies = spec.frequencies if spec.frequencies is not None else inverse_frequencies(spec.rotary_dim, spec.theta)
+        self.inv_freq = torch.tensor(list(frequencies), dtype=torch.float64, device=device)
+        self.magnitude = float(getattr(spec, "magnitude", 1.0))
+
+    def pair_tables(self, ctx):
+        """(cos, sin): float32 [T, rotary_dim/2] each, for the rows of this step; pair i is turned by angle i."""
+        key = ("rotary_interleaved", self.spec)
+        if key not in ctx.memo:
+            cos = torch.empty((ctx.n_rows, self.rotary_dim // 2), dtype=torch.float32, device=ctx.device)
+            sin = torch.empty_like(cos)
+            ops.rope_cos_sin(ctx.row_pos, self.inv_freq, cos, sin, self.magnitude)
+            ctx.memo[key] = (cos, sin)
+        return ctx.memo[key]
 
 
 def rotation_tables(position, ctx):
@@ -75,3 +100,4 @@ def rotation_tables(position, ctx):
 
 register_position_encoding("rotary_half_split", RotaryHalfSplit)
 register_position_encoding("rotary_partial", RotaryPartial)
+register_position_encoding("rotary_interleaved", RotaryInterleaved)
