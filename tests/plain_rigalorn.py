@@ -11,6 +11,9 @@ A Rigalorn layer is "parallel": with h = norm(x), x <- x + mixer(h) + feed_forwa
   latent_attention   queries and keys/values through low-rank latents; one rotated key part shared by all heads (pairs 2i,
                      2i + 1), a sliding window.
 The feed-forward is down(act(up(h))) with a two-parameter activation that is quadratic on the right and exponential on the left.
+
+`store`, where a function takes it, is applied to what an engine that computes in bfloat16 would keep in bfloat16 (rows that go
+into a matrix product, cached keys and values); the identity by default.  It serves to measure what such rounding alone does.
 """
 from __future__ import annotations
 
@@ -34,8 +37,16 @@ def xielu(z, p, q):
     return torch.where(z > 0, right, left)
 
 
-def dense_mlp(h, up, down, act):
-    return xielu(h @ up.T, act[0], act[1]) @ down.T
+def same(x):
+    return x
+
+
+def to_bfloat16_and_back(x):
+    return x.to(torch.bfloat16).to(x.dtype)
+
+
+def dense_mlp(h, up, down, act, store=same):
+    return store(xielu(h @ up.T, act[0], act[1])) @ down.T
 
 
 def rotary_frequencies(dims, base, scaling=None):
@@ -99,7 +110,7 @@ def softmax_attention(q, k, v, scale, window):
     return torch.einsum("hts,shd->thd", torch.softmax(scores, dim=-1), v)
 
 
-def attention(h, w, m, v_first=None):
+def attention(h, w, m, v_first=None, store=same):
     """m: the layer's `mixer` entry of config.json; w: its tensors by their short names.  Returns (output, the values it used
     before blending if it is the first blending layer, else None)."""
     T = h.shape[0]
@@ -118,25 +129,25 @@ def attention(h, w, m, v_first=None):
             lam = w["vmix"]
             v = (1 - lam) * v + lam * v_first
     window = m["mask"]["size"] if m.get("mask") else None
-    o = softmax_attention(q, k, v, m["scale"], window)
-    return o.reshape(T, H * dv) @ w["o"].T, own
+    o = softmax_attention(store(q), store(k), store(v), m["scale"], window)
+    return store(o.reshape(T, H * dv)) @ w["o"].T, own
 
 
-def latent_attention(h, w, m, eps):
+def latent_attention(h, w, m, eps, store=same):
     T = h.shape[0]
     H, d, r, dv, rank = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
-    cq = rms_norm(h @ w["dq"].T, w["dq.norm"], eps)
+    cq = store(rms_norm(h @ w["dq"].T, w["dq.norm"], eps))
     q = (cq @ w["uq"].T).view(T, H, d + r)
     down = h @ w["dkv"].T
-    c = rms_norm(down[:, :rank], w["dkv.norm"], eps)
+    c = store(rms_norm(down[:, :rank], w["dkv.norm"], eps))
     f, _ = rotary_frequencies(r, m["rot"]["base"])
-    k_rot = rotate_interleaved(down[:, None, rank:], f)                     # [T, 1, r], one for all heads
-    q_rot = rotate_interleaved(q[..., d:], f)
+    k_rot = store(rotate_interleaved(down[:, None, rank:], f))              # [T, 1, r], one for all heads
+    q_rot = store(rotate_interleaved(q[..., d:], f))
     k = torch.cat([(c @ w["uk"].T).view(T, H, d), k_rot.expand(T, H, r)], dim=-1)
     v = (c @ w["uv"].T).view(T, H, dv)
     window = m["mask"]["size"] if m.get("mask") else None
-    o = softmax_attention(torch.cat([q[..., :d], q_rot], dim=-1), k, v, m["scale"], window)
-    return o.reshape(T, H * dv) @ w["o"].T
+    o = softmax_attention(torch.cat([store(q[..., :d]), q_rot], dim=-1), k, v, m["scale"], window)
+    return store(o.reshape(T, H * dv)) @ w["o"].T
 
 
 def short_conv_silu(x, taps):
@@ -160,7 +171,7 @@ def delta_rule(q, k, v, beta, g):
     return torch.stack(out)
 
 
-def delta(h, w, m, eps):
+def delta(h, w, m, eps, store=same):
     T = h.shape[0]
     H, G, dk, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     q = short_conv_silu(h @ w["q"].T, w["q.conv"]).view(T, G, dk)
@@ -176,10 +187,10 @@ def delta(h, w, m, eps):
         o = delta_rule(q[:, j], k[:, j], v[:, i], beta[:, i], g[:, i])
         heads.append(o / torch.sqrt((o * o).mean(dim=-1, keepdim=True) + eps) * w["norm"])
     gate = h @ w["g"].T
-    return (torch.cat(heads, dim=-1) * (gate * torch.sigmoid(gate))) @ w["o"].T
+    return store(torch.cat(heads, dim=-1) * (gate * torch.sigmoid(gate))) @ w["o"].T
 
 
-def forward(config, tensors, tokens, dtype=torch.float64, layer_outputs=None):
+def forward(config, tensors, tokens, dtype=torch.float64, layer_outputs=None, store=same):
     """Logits [T, vocab] of a whole sequence.  config: config.json as a dict; tensors: by name.  layer_outputs: a list that
     gets the residual stream after every layer."""
     t = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in tensors.items()}
@@ -189,20 +200,28 @@ def forward(config, tensors, tokens, dtype=torch.float64, layer_outputs=None):
     for i, layer in enumerate(config["layers"]):
         p = f"l{i}."
         w = {k[len(p) + 4:]: v for k, v in t.items() if k.startswith(p + "mix.")}
-        h = rms_norm(x, t[p + "norm1"], eps)
+        h = store(rms_norm(x, t[p + "norm1"], eps))
         kind, m = layer["type"], layer["mixer"]
         if kind == "attention":
-            mixed, own = attention(h, w, m, v_first)
+            mixed, own = attention(h, w, m, v_first, store)
             v_first = own if own is not None else v_first
         elif kind == "latent_attention":
-            mixed = latent_attention(h, w, m, eps)
+            mixed = latent_attention(h, w, m, eps, store)
         elif kind == "delta":
-            mixed = delta(h, w, m, eps)
+            mixed = delta(h, w, m, eps, store)
         else:
             raise ValueError(f"unknown layer type {kind!r}")
         if layer.get("mlp") is not None:
-            mixed = mixed + dense_mlp(h, t[p + "mlp.up"], t[p + "mlp.down"], t[p + "mlp.act"])
+            mixed = mixed + dense_mlp(h, t[p + "mlp.up"], t[p + "mlp.down"], t[p + "mlp.act"], store)
         x = x + mixed
         if layer_outputs is not None:
             layer_outputs.append(x)
-    return rms_norm(x, t["final.norm"], eps) @ t["head"].T
+    return store(rms_norm(x, t["final.norm"], eps)) @ t["head"].T
+
+
+def greedy(config, tensors, prompt, n, dtype=torch.float64):
+    """The n tokens that follow `prompt` when the likeliest is taken every time (the lowest index on ties)."""
+    tokens = list(prompt)
+    for _ in range(n):
+        tokens.append(int(torch.argmax(forward(config, tensors, tokens, dtype)[-1])))
+    return tokens[len(prompt):]

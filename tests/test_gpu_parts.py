@@ -160,9 +160,9 @@ def test_a_mixer_of_ones_own_uses_the_attention_front_half_with_a_hook(dtype):
 def test_attention_refuses_a_head_size_its_kernels_do_not_take():
     from geneinfer_amd.config import AttentionSpec
     from geneinfer_amd.parts import mixer_class
-    spec = AttentionSpec(64, 1, 1, 272, "q", "k", "v", "o")
-    w = {"q": torch.zeros(272, 64, device=DEV), "k": torch.zeros(272, 64, device=DEV), "v": torch.zeros(272, 64, device=DEV), "o": torch.zeros(64, 272, device=DEV)}
-    with pytest.raises(ValueError, match="head_dim = 272"):
+    spec = AttentionSpec(64, 1, 1, 656, "q", "k", "v", "o")
+    w = {"q": torch.zeros(656, 64, device=DEV), "k": torch.zeros(656, 64, device=DEV), "v": torch.zeros(656, 64, device=DEV), "o": torch.zeros(64, 656, device=DEV)}
+    with pytest.raises(ValueError, match="head_dim = 656"):
         mixer_class(spec)(spec, w, torch.float32, DEV)
 
 
