@@ -2,6 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--config FILE] [--prefill-tokens T] [--layers L] [--no-points]
     python bench.py --fekorax [--sizes 1b,8b] [--layers L] [--batch B] [--prefill-tokens T]     (another record: see `fekorax_beside_llama`)
+    python bench.py --rigalorn [--sizes 1b,8b] [--layers L] [--batch B] [--prefill-tokens T]    (another record: see `rigalorn_beside_fekorax`)
 
 A step is one decode step of the whole batch (default batch 8, each request on a 2,048-token
 prompt in a 4,096-token context), through the scheduler with its defaults.  After W warm-up steps,
@@ -72,51 +73,104 @@ def fekorax_beside_llama(args) -> int:
                        max_positions=T + 1024)
         record["sizes"][size] = {}
         for name, cfg in (("llama", llama), ("fekorax", fekorax)):
-            model = random_model(parse_config(cfg), seed=0, dtype="bfloat16" if args.dtype == "bf16" else "float32", device="cuda:0", draw_on_device=True)
-            runner = Runner(model, page_size=PAGE, max_tokens=batch * (T + 512), max_requests=batch, max_rows=max(T, batch), max_positions=T + 1024)
-            prompts = [torch.randint(0, vocab, (T,), generator=gen).tolist() for _ in range(batch)]
+            record["sizes"][size][name] = _measure_design(cfg, args, T, batch, steps, vocab, gen)
+    print(json.dumps(record))
+    return 0
 
-            def prefill_all():
-                times = []
-                for r, p in enumerate(prompts):
-                    if runner.is_open(r):
-                        runner.close(r)
-                    runner.open(r)
-                    torch.cuda.synchronize()
-                    t0 = time.perf_counter()
-                    runner.step([StepEntry(r, p, (T - 1,))])
-                    torch.cuda.synchronize()
-                    times.append(time.perf_counter() - t0)
-                return sorted(times)[len(times) // 2]
 
-            def decode_steps(n):
-                entries = [StepEntry(r, [7], (0,)) for r in range(batch)]
-                torch.cuda.synchronize()
-                t0 = time.perf_counter()
-                for _ in range(n):
-                    runner.step(entries)
-                torch.cuda.synchronize()
-                return (time.perf_counter() - t0) / n
+def _measure_design(cfg, args, T, batch, steps, vocab, gen) -> dict:
+    """Prefill of one prompt of T tokens (median over `batch` prompts), decode steps of the batch on those contexts (captured), and
+    the time of every kernel in both (the device waited for around each)."""
+    import torch
+    from geneinfer_amd.config import parse_config
+    from geneinfer_amd.engine import Runner, StepEntry, random_model
+    from geneinfer_amd.kernels import ops
+    model = random_model(parse_config(cfg), seed=0, dtype="bfloat16" if args.dtype == "bf16" else "float32", device="cuda:0", draw_on_device=True)
+    runner = Runner(model, page_size=PAGE, max_tokens=batch * (T + 512), max_requests=batch, max_rows=max(T, batch), max_positions=T + 1024)
+    prompts = [torch.randint(0, vocab, (T,), generator=gen).tolist() for _ in range(batch)]
 
-            prefill_all()
-            prefill_s = prefill_all()
-            decode_steps(args.warmup)
-            decode_s = sorted(decode_steps(steps) for _ in range(3))[1]
-            # the same once more with every kernel timed (no captured steps meanwhile)
-            by_kernel = {}
-            for what, run in (("prefill", lambda: (runner.close(0), runner.open(0), runner.step([StepEntry(0, prompts[0], (T - 1,))]))),
-                              ("decode", lambda: decode_steps(4))):
-                profile = ops.set_profiling(True)
-                run()
-                torch.cuda.synchronize()
-                n = 1 if what == "prefill" else 4
-                by_kernel[what] = {k: [profile.calls[k] // n, round(v * 1e3 / n, 4)] for k, v in sorted(profile.seconds.items(), key=lambda kv: -kv[1])}
-                ops.set_profiling(False)
-            record["sizes"][size][name] = {"prefill_tok_s": round(T / prefill_s, 1), "prefill_ms": round(prefill_s * 1e3, 3), "decode_ms_per_step": round(decode_s * 1e3, 4),
-                                           "decode_tok_s": round(batch / decode_s, 1), "weight_bytes_per_step": model.weight_bytes_read_per_step(),
-                                           "kernels_calls_ms": by_kernel}
-            del runner, model
-            torch.cuda.empty_cache()
+    def prefill_all():
+        times = []
+        for r, p in enumerate(prompts):
+            if runner.is_open(r):
+                runner.close(r)
+            runner.open(r)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            runner.step([StepEntry(r, p, (T - 1,))])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+        return sorted(times)[len(times) // 2]
+
+    def decode_steps(n):
+        entries = [StepEntry(r, [7], (0,)) for r in range(batch)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            runner.step(entries)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n
+
+    prefill_all()
+    prefill_s = prefill_all()
+    decode_steps(args.warmup)
+    decode_s = sorted(decode_steps(steps) for _ in range(3))[1]
+    # the same once more with every kernel timed (no captured steps meanwhile)
+    by_kernel = {}
+    for what, run in (("prefill", lambda: (runner.close(0), runner.open(0), runner.step([StepEntry(0, prompts[0], (T - 1,))]))),
+                      ("decode", lambda: decode_steps(4))):
+        profile = ops.set_profiling(True)
+        run()
+        torch.cuda.synchronize()
+        n = 1 if what == "prefill" else 4
+        by_kernel[what] = {k: [profile.calls[k] // n, round(v * 1e3 / n, 4)] for k, v in sorted(profile.seconds.items(), key=lambda kv: -kv[1])}
+        ops.set_profiling(False)
+    result = {"prefill_tok_s": round(T / prefill_s, 1), "prefill_ms": round(prefill_s * 1e3, 3), "decode_ms_per_step": round(decode_s * 1e3, 4),
+              "decode_tok_s": round(batch / decode_s, 1), "weight_bytes_per_step": model.weight_bytes_read_per_step(), "kernels_calls_ms": by_kernel}
+    del runner, model
+    torch.cuda.empty_cache()
+    return result
+
+
+def rigalorn_beside_fekorax(args) -> int:
+    """The Rigalorn design at layer shapes of real models beside the Fekorax design (the nearest the engine has: memories and
+    attention in turns) and the Llama decoder at the same shapes, random weights; measured as `fekorax_beside_llama` measures.  A
+    Rigalorn model of L layers here is L/4 times [gated delta rule; attention through latents; attention with blended values;
+    gated delta rule], every layer with its feed-forward beside the mixer: the attention with the Llama layer's heads (biases,
+    rotation of half of each head with stretched frequencies, a window of 1,024), the latents of 4 and 12 head sizes for keys/values
+    and queries with half a head size of rotated channels, the memories with a quarter as many heads of the same key size and twice
+    the value size (as Fekorax's here), convolutions of 4 taps.  One JSON line."""
+    import torch
+    T, batch, L, steps = args.prefill_tokens, args.batch, args.layers or 8, args.steps
+    gen = torch.Generator().manual_seed(1)
+    record = {"metric": "Rigalorn beside Fekorax and Llama at equal layer shapes: prefill tok/s, decode ms a step, ms by kernel", "dtype": args.dtype, "layers": L,
+              "prefill_tokens": T, "decode_batch": batch, "data": "synthetic: random weights by formula, uniform random token ids", "sizes": {}}
+    for size in args.sizes.split(","):
+        D, H, G, hd, ff, vocab = FEKORAX_SIZES[size]
+        mlp = dict(kind="dense", ff=ff)
+        llama = dict(architectures=["LlamaForCausalLM"], hidden_size=D, intermediate_size=ff, num_hidden_layers=L, num_attention_heads=H,
+                     num_key_value_heads=G, head_dim=hd, vocab_size=vocab, max_position_embeddings=T + 1024, rope_theta=500000.0, rms_norm_eps=1e-5,
+                     tie_word_embeddings=True)
+        att = lambda source=None: dict(type="attention", mlp=mlp, mixer=dict(
+            heads=H, kv_heads=G, dim=hd, vdim=hd, scale=hd ** -0.5, rot=dict(dims=hd // 2, base=10000.0), mask=dict(size=1024),
+            **({} if source is None else dict(kv_from=source))))
+        mem = dict(type="mlstm", mlp=None, mixer=dict(heads=max(1, H // 4), dim=hd, vdim=2 * hd, gate_cap=12.0))
+        layers = []
+        for i in range(0, L, 4):
+            layers += [mem, att(), mem, att(i + 1)]
+        fekorax = dict(architecture="Fekorax", vocab=vocab, width=D, embedding=dict(scale=D ** 0.5), norm=dict(eps=1e-5), layers=layers[:L], max_positions=T + 1024)
+        delta = dict(type="delta", mlp=mlp, mixer=dict(heads=max(1, H // 4), kv_heads=max(1, H // 8), dim=hd, vdim=2 * hd, conv=4))
+        latent = dict(type="latent_attention", mlp=mlp, mixer=dict(heads=H, dim=hd, rot_dim=hd // 2, vdim=hd, q_rank=12 * hd, kv_rank=4 * hd, scale=(1.5 * hd) ** -0.5,
+                                                                    rot=dict(dims=hd // 2, base=1e6), mask=dict(size=1024)))
+        blended = dict(type="attention", mlp=mlp, mixer=dict(heads=H, kv_heads=G, dim=hd, vdim=hd, scale=hd ** -0.5, v_mix=True, mask=dict(size=1024), rot=dict(
+            dims=hd // 2, base=10000.0, scaling=dict(factor=8.0, original=1024, fast=32.0, slow=1.0))))
+        rigalorn = dict(architecture="Rigalorn", vocab=vocab, width=D, embedding=dict(scale=D ** 0.5), norm=dict(eps=1e-5), max_positions=T + 1024,
+                        layers=([delta, latent, blended, delta] * ((L + 3) // 4))[:L])
+        record["sizes"][size] = {}
+        for name, cfg in (("llama", llama), ("fekorax", fekorax), ("rigalorn", rigalorn)):
+            if args.only and name not in args.only.split(","):
+                continue
+            record["sizes"][size][name] = _measure_design(cfg, args, T, batch, steps, vocab, gen)
     print(json.dumps(record))
     return 0
 
@@ -133,7 +187,9 @@ def main() -> int:
     ap.add_argument("--config", default="", help="a config.json of another size of the architecture (default: the Llama-3.2-1B shape)")
     ap.add_argument("--prefill-tokens", type=int, default=PROMPT, help="length of the timed prompt")
     ap.add_argument("--fekorax", action="store_true", help="another measurement: the Fekorax design beside Llama at equal layer shapes (see fekorax_beside_llama)")
-    ap.add_argument("--sizes", default="1b,8b", help="with --fekorax: layer shapes, of " + ", ".join(FEKORAX_SIZES))
+    ap.add_argument("--rigalorn", action="store_true", help="another measurement: the Rigalorn design beside Fekorax and Llama at equal layer shapes (see rigalorn_beside_fekorax)")
+    ap.add_argument("--only", default="", help="with --rigalorn: the designs to measure, of llama, fekorax, rigalorn (default: all)")
+    ap.add_argument("--sizes", default="1b,8b", help="with --fekorax or --rigalorn: layer shapes, of " + ", ".join(FEKORAX_SIZES))
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine")
@@ -141,6 +197,8 @@ def main() -> int:
 
     if args.fekorax:
         return fekorax_beside_llama(args)
+    if args.rigalorn:
+        return rigalorn_beside_fekorax(args)
 
     import torch
     from geneinfer_amd.config import LlamaConfig

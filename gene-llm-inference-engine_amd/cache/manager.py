@@ -51,7 +51,7 @@ class PageGroup:
         self.storage = None
         self.table_dev = None
         if allocate_storage:
-            if (need.value_dim is None or need.value_dim == need.head_dim) and not getattr(need, "values_in_keys", False):
+            if need.value_dim is None or need.value_dim == need.head_dim:
                 self.storage = torch.zeros((len(entries), n_pages + 1, 2, need.n_kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
             else:         # keys [kv_head][place][head_dim], then values [kv_head][value_dim][place]: a page is one run of numbers
                 self.storage = torch.zeros((len(entries), n_pages + 1, page_size * need.elements_per_position()), dtype=dtype, device=device)

@@ -11,18 +11,14 @@ import torch
 class PagedKvNeed:
     """Keys and values of every position (or of the last `window` positions, or of the positions of the chunk of `chunk`
     positions that the request is in: what no later position can see is given back) in pages.  `value_dim`: channels of a
-    value head where they differ from a key head's `head_dim`.  `values_in_keys`: nothing is stored for the values, which are
-    the first `value_dim` channels of the keys (a latent that serves as both); a page is then [kv_head][place][head_dim]."""
+    value head where they differ from a key head's `head_dim`."""
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     value_dim: Optional[int] = None
     chunk: Optional[int] = None
-    values_in_keys: bool = False
 
     def elements_per_position(self) -> int:
-        if self.values_in_keys:
-            return self.n_kv_heads * self.head_dim
         return self.n_kv_heads * (self.head_dim + (self.value_dim or self.head_dim))
 
     def first_visible(self, position: int) -> int:

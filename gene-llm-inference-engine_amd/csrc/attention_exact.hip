@@ -18,8 +18,7 @@
 //
 // Cache of one layer: per page the keys [kv_head][place][hd], then the values transposed
 // [kv_head][vd][place] (vd channels a value head, hd a key head); table[slot][i] is the page of
-// positions i*page_size .. (i+1)*page_size - 1.  With `v_in_k` a page holds keys only and a position's value is the first vd
-// channels of its key (attention over a latent that serves as key and value alike: no second copy is kept).
+// positions i*page_size .. (i+1)*page_size - 1.
 #include "common.h"
 
 namespace {
@@ -31,7 +30,7 @@ __global__ __launch_bounds__(64) void attention_exact_kernel(const TQ* __restric
                                                             const int* __restrict__ pos, const int* __restrict__ slot,
                                                             const int* __restrict__ table, int table_stride, long page_stride,
                                                             int page_size, int n_heads, int n_kv, int hd, int vd, int window, int chunk, float scale,
-                                                            const float* __restrict__ sinks, const float* __restrict__ gate, long gate_stride, int v_in_k) {
+                                                            const float* __restrict__ sinks, const float* __restrict__ gate, long gate_stride) {
     __shared__ float q_s[MAX_HD];
     __shared__ float p_s[64];
     __shared__ long v_off[64];
@@ -45,7 +44,6 @@ __global__ __launch_bounds__(64) void attention_exact_kernel(const TQ* __restric
     __syncthreads();
 
     const long v_plane = (long)n_kv * page_size * hd;   // from a page's keys to its values
-    const long v_step = v_in_k ? 1 : page_size;         // from one channel of a position's value to the next
     float m = sinks ? sinks[h] : -INFINITY;
     double l = sinks ? 1.0 : 0.0;
     float acc[MAX_HD / 64] = {};
@@ -57,7 +55,7 @@ __global__ __launch_bounds__(64) void attention_exact_kernel(const TQ* __restric
         if (valid) {
             const long page = (long)tab[j / page_size] * page_stride;
             off = page + ((long)g * page_size + j % page_size) * hd;
-            voff = v_in_k ? off : page + v_plane + (long)g * vd * page_size + j % page_size;
+            voff = page + v_plane + (long)g * vd * page_size + j % page_size;
             float dot = 0.f;
             for (int d = 0; d < hd; ++d) dot = fmaf(q_s[d], load_f32(cache, off + d), dot);
             s = dot * scale;
@@ -80,7 +78,7 @@ __global__ __launch_bounds__(64) void attention_exact_kernel(const TQ* __restric
 #pragma unroll
             for (int i = 0; i < MAX_HD / 64; ++i) {
                 const int d = lane + 64 * i;
-                if (d < vd) acc[i] = fmaf(pj, load_f32(cache, vo + (long)d * v_step), acc[i]);
+                if (d < vd) acc[i] = fmaf(pj, load_f32(cache, vo + (long)d * page_size), acc[i]);
             }
         }
     }
@@ -100,19 +98,18 @@ GI_API int gi_attention_exact_max_head_size() { return MAX_HD; }
 GI_API int gi_attention_exact(const void* q, int q_dtype, const void* cache, int cache_dtype, void* out, int out_dtype, const int* pos,
                               const int* slot, const int* table, int table_stride, long page_stride, int page_size, int n_rows,
                               int n_heads, int n_kv, int hd, int vd, int window, int chunk, float scale, const float* sinks, const float* gate,
-                              long gate_stride, int v_in_k, hipStream_t stream) {
+                              long gate_stride, hipStream_t stream) {
     GI_REQUIRE(n_rows > 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attention_exact: bad head counts (%d rows, %d heads, %d kv heads)",
                n_rows, n_heads, n_kv);
     GI_REQUIRE(hd > 0 && hd <= MAX_HD, "attention_exact: head size %d is outside 1..%d", hd, MAX_HD);
     GI_REQUIRE(vd > 0 && vd <= MAX_HD, "attention_exact: value head size %d is outside 1..%d", vd, MAX_HD);
     GI_REQUIRE(window >= 0 && chunk >= 0 && (gate == nullptr || gate_stride >= n_heads), "attention_exact: bad window, chunk or gate stride");
-    GI_REQUIRE(page_size > 0 && page_stride >= (long)n_kv * page_size * (hd + (v_in_k ? 0 : vd)), "attention_exact: page stride %ld too small", page_stride);
-    GI_REQUIRE(!v_in_k || vd <= hd, "attention_exact: values taken from the keys cannot be longer than the keys (%d > %d)", vd, hd);
+    GI_REQUIRE(page_size > 0 && page_stride >= (long)n_kv * page_size * (hd + vd), "attention_exact: page stride %ld too small", page_stride);
     GI_REQUIRE((long)n_rows * n_heads < 2147483647L, "attention_exact: too many (row, head) pairs");
     const unsigned grid = (unsigned)(n_rows * n_heads);
 #define GO(TQ, TC, TO)                                                                                                          \
     attention_exact_kernel<TQ, TC, TO><<<grid, 64, 0, stream>>>((const TQ*)q, (const TC*)cache, (TO*)out, pos, slot, table, table_stride, \
-                                                                page_stride, page_size, n_heads, n_kv, hd, vd, window, chunk, scale, sinks, gate, gate_stride, v_in_k)
+                                                                page_stride, page_size, n_heads, n_kv, hd, vd, window, chunk, scale, sinks, gate, gate_stride)
     if (q_dtype == GI_F32 && cache_dtype == GI_F32 && out_dtype == GI_F32) GO(float, float, float);
     else if (q_dtype == GI_BF16 && cache_dtype == GI_BF16 && out_dtype == GI_BF16) GO(bf16_t, bf16_t, bf16_t);
     else return gi_fail("attention_exact: dtypes (%d, %d, %d) must be all float32 or all bfloat16", q_dtype, cache_dtype, out_dtype);

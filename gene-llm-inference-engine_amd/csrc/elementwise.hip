@@ -541,22 +541,30 @@ GI_API int gi_act_mul(const float* gate_up, void* h, int h_dtype, int n_rows, in
 __device__ __forceinline__ float softplus_f32(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 
 template <typename TO>
-__global__ void xielu_kernel(const float* __restrict__ x, long ldx, TO* __restrict__ h, long ldh, int inter, size_t n, const float* __restrict__ params) {
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
-    const size_t t = i / inter, c = i % inter;
+__global__ __launch_bounds__(256) void xielu_kernel(const float* __restrict__ x, long ldx, TO* __restrict__ h, long ldh, int inter, const float* __restrict__ params) {
+    // one row a workgroup (blockIdx.x) and 1,024 columns of it (blockIdx.y): four neighbouring columns a thread where the row allows
     const float a = softplus_f32(params[0]), b = 0.5f + softplus_f32(params[1]);
-    const float z = x[t * ldx + c];
-    const float y = z > 0.f ? fmaf(a * z, z, 0.5f * z) : fmaf(b, expm1f(z) - z, 0.5f * z);
-    store_f32(h, t * ldh + c, y);
+    const float* xr = x + (size_t)blockIdx.x * ldx;
+    TO* hr = h + (size_t)blockIdx.x * ldh;
+    auto act = [&](float z) { return z > 0.f ? fmaf(a * z, z, 0.5f * z) : fmaf(b, expm1f(z) - z, 0.5f * z); };
+    const int c0 = blockIdx.y * 1024 + threadIdx.x * 4;
+    if (c0 + 3 < inter && (ldx & 3) == 0 && (((uintptr_t)x) & 15) == 0) {
+        const float4 z = *reinterpret_cast<const float4*>(xr + c0);
+        store_f32(hr, c0, act(z.x));
+        store_f32(hr, c0 + 1, act(z.y));
+        store_f32(hr, c0 + 2, act(z.z));
+        store_f32(hr, c0 + 3, act(z.w));
+    } else {
+        for (int c = c0; c < min(c0 + 4, inter); ++c) store_f32(hr, c, act(xr[c]));
+    }
 }
 
 GI_API int gi_xielu(const float* x, long ldx, void* h, int h_dtype, long ldh, int n_rows, int inter, const float* params, hipStream_t stream) {
     GI_REQUIRE(n_rows > 0 && inter > 0 && ldx >= inter && ldh >= inter && params != nullptr, "xielu: bad sizes (rows %d, columns %d) or no parameters", n_rows, inter);
-    const size_t n = (size_t)n_rows * inter;
-    const unsigned blocks = (unsigned)((n + 255) / 256);
-    if (h_dtype == GI_F32) xielu_kernel<float><<<blocks, 256, 0, stream>>>(x, ldx, (float*)h, ldh, inter, n, params);
-    else if (h_dtype == GI_BF16) xielu_kernel<bf16_t><<<blocks, 256, 0, stream>>>(x, ldx, (bf16_t*)h, ldh, inter, n, params);
+    GI_REQUIRE((inter + 1023) / 1024 <= 65535, "xielu: rows too long");
+    dim3 grid(n_rows, (inter + 1023) / 1024);
+    if (h_dtype == GI_F32) xielu_kernel<float><<<grid, 256, 0, stream>>>(x, ldx, (float*)h, ldh, inter, params);
+    else if (h_dtype == GI_BF16) xielu_kernel<bf16_t><<<grid, 256, 0, stream>>>(x, ldx, (bf16_t*)h, ldh, inter, params);
     else return gi_fail("xielu: unknown dtype %d", h_dtype);
     GI_CHECK_LAUNCH("xielu");
     return 0;

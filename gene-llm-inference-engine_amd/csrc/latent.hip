@@ -2,16 +2,22 @@
 //
 // A layer of this kind projects a row down twice: to a query latent of `q_rank` numbers, and to a key/value latent of `kv_rank`
 // numbers with `rot` more that are one rotated key part for all heads.  Both latents are RMS-normed with weights of their own.
-// Only the normed key/value latent c and the rotated part are cached: a page holds, per place, one "key" [kv_rank + rot] and
-// nothing else, because with the up projections folded into the query (q' = W_uk^T q per head) and into the output
-// (o = W_uv sum_j p_j c_j) the latent is key and value at once:
+// Only the normed key/value latent c and the rotated part are cached, nothing per head, because with the up projections folded
+// into the query (q' = W_uk^T q per head) and into the output (o = W_uv sum_j p_j c_j) the latent is key and value at once:
 //     score_j = q' . c_j + q_rot . k_rot_j          out = sum_j softmax(score)_j c_j
+// A page holds its places' keys [place][kv_rank + rot] and, behind them, the latent once more with the places innermost
+// [kv_rank][place]: the layout of a layer with one key/value head whose values are shorter than its keys, which every attention
+// kernel reads, and both operands of the matrix instructions come out of memory as they lie.
 // The rotation here turns neighbouring channels, the pair (2i, 2i + 1) by pos * f_i.
 //
 //   latent_prepare   one wave per (row, which): the query latent normed into the rows the up projection reads; the key/value
 //                    latent normed and the rotated part turned, both written to the row's place in its page
 //   latent_queries   one wave per (row, head): a head's unrotated channels into the rows the folding product reads, its
 //                    rotated channels turned and written behind the place where that product puts q'
+//   heads_product    out[t, h, :] = a[t, h, :] W_h^T for every head in one launch (the folding of W_uk into the queries and the
+//                    product with W_uv behind the attention), on the matrix cores
+//   latent_attention one wave per (row, 16 heads, share of the context): all heads read the same keys, so 16 of them are the
+//                    columns of one matrix instruction even for a single decoded row
 #include "common.h"
 
 namespace {
@@ -38,7 +44,12 @@ __global__ __launch_bounds__(64) void latent_prepare_kernel(const float* __restr
     const int p = pos[t];
     const long page = table[(size_t)slot[t] * table_stride + p / page_size];
     TC* dst = cache + page * page_stride + (size_t)(p % page_size) * (kv_rank + rot);
-    for (int d = lane; d < n; d += 64) store_f32(dst, d, load_f32(w, d) * (r * src[d]));
+    TC* as_value = cache + page * page_stride + (size_t)page_size * (kv_rank + rot) + p % page_size;      // [kv_rank][place]
+    for (int d = lane; d < n; d += 64) {
+        const float c = load_f32(w, d) * (r * src[d]);
+        store_f32(dst, d, c);
+        store_f32(as_value, (size_t)d * page_size, c);
+    }
     for (int i = lane; i < rot / 2; i += 64) {
         const float u = src[kv_rank + 2 * i], v = src[kv_rank + 2 * i + 1];
         const float c = cos_t[(size_t)t * (rot / 2) + i], s = sin_t[(size_t)t * (rot / 2) + i];
@@ -63,17 +74,204 @@ __global__ __launch_bounds__(64) void latent_queries_kernel(const float* __restr
     }
 }
 
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// out[t, h*n_out + n] = sum_k a[t, h*k_dim + k] * w[h][n][k], bfloat16 operands, 32-bit sums.  One wave per (16 rows, head, 64
+// columns): the operands of the 16x16x32 matrix instruction are 16-byte pieces of a's and w's rows as they lie in memory.
+template <typename TO>
+__global__ __launch_bounds__(64) void heads_product_kernel(const bf16_t* __restrict__ a, long lda, const bf16_t* __restrict__ w, TO* __restrict__ out, long ldo,
+                                                          long out_head_stride, int n_rows, int k_dim, int n_out) {
+    const int lane = threadIdx.x, r = lane & 15, q4 = lane >> 4;
+    const int row0 = blockIdx.x * 16, h = blockIdx.y, col0 = blockIdx.z * 64;
+    const int row = min(row0 + r, n_rows - 1);
+    const bf16_t* arow = a + (size_t)row * lda + (size_t)h * k_dim;
+    const bf16_t* wh = w + (size_t)h * n_out * k_dim;
+    floatx4 acc[4] = {floatx4{}, floatx4{}, floatx4{}, floatx4{}};
+    for (int k0 = 0; k0 < k_dim; k0 += 32) {
+        const int k = k0 + 8 * q4;
+        const bool in = k < k_dim;                       // (k_dim is a multiple of 8: a piece is inside or outside as a whole)
+        uint4 av = *reinterpret_cast<const uint4*>(arow + (in ? k : 0));
+        if (!in) av = uint4{0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int col = min(col0 + 16 * j + r, n_out - 1);
+            uint4 wv = *reinterpret_cast<const uint4*>(wh + (size_t)col * k_dim + (in ? k : 0));
+            if (!in) wv = uint4{0, 0, 0, 0};
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(av), as_bf16x8(wv), acc[j], 0, 0, 0);
+        }
+    }
+    // element v of acc[j]: row row0 + 4*q4 + v, column col0 + 16*j + r
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int col = col0 + 16 * j + r;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int t = row0 + 4 * q4 + v;
+            if (t < n_rows && col < n_out) store_f32(out, (size_t)t * ldo + (size_t)h * out_head_stride + col, acc[j][v]);
+        }
+    }
+}
+
+// Attention over the latent pages on the matrix cores.  One wave: row t, heads 16 hg .. 16 hg + 15, share `sp` of the row's
+// context.  Tiles of 32 positions (two blocks of 16, each inside one page): S^T = K Q^T puts a position's scores for the 16 heads
+// into one lane group, so that a head's maximum and sum are a lane's own plus two exchanges; the probabilities, as they lie, are
+// the second operand of O^T = V^T P^T.  KS = key channels / 32 (rounded up: pieces beyond the key are zeros), DT = value channels / 16.
+// Shares of one row meet in `part` ([row][head][share]{m, l, o[vd]}, 32-bit) and `latent_merge_kernel` adds them; with one share
+// the wave writes the heads' outputs itself.
+template <int KS, int DT>
+__global__ __launch_bounds__(64) void latent_attention_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache, bf16_t* __restrict__ out,
+                                                             float* __restrict__ part, const int* __restrict__ pos, const int* __restrict__ slot,
+                                                             const int* __restrict__ table, int table_stride, long page_stride, int page_size,
+                                                             int n_heads, int kd, int vd, int window, float scale2, int n_splits) {
+    const int lane = threadIdx.x, r = lane & 15, q4 = lane >> 4;
+    const int t = blockIdx.x, hg = blockIdx.y, sp = blockIdx.z;
+    const int head = hg * 16 + r;
+    const bool head_ok = head < n_heads;
+    const int p = pos[t];
+    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int* tab = table + (size_t)slot[t] * table_stride;
+    // this share's tiles
+    const int first_tile = lo >> 5, n_tiles = (p >> 5) - first_tile + 1;
+    const int per = (n_tiles + n_splits - 1) / n_splits;
+    const int tile0 = first_tile + sp * per, tile1 = min(tile0 + per, first_tile + n_tiles);
+    const long v_plane = (long)page_size * kd;
+
+    bf16x8 qreg[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        const int c = 32 * ks + 8 * q4;
+        uint4 v = *reinterpret_cast<const uint4*>(q + ((size_t)t * n_heads + (head_ok ? head : 0)) * kd + (c < kd ? c : 0));
+        if (!head_ok || c >= kd) v = uint4{0, 0, 0, 0};
+        qreg[ks] = as_bf16x8(v);
+    }
+    floatx4 o[DT];
+#pragma unroll
+    for (int i = 0; i < DT; ++i) o[i] = floatx4{};
+    float m = -INFINITY, l = 0.f;
+
+    for (int tile = tile0; tile < tile1; ++tile) {
+        const int kv0 = tile << 5;
+        const bf16_t* page[2];
+        int place[2];
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {                    // a block that lies outside what the row sees is read from a place that it does see
+            const int j0 = min(max(kv0 + 16 * b, lo & ~15), p & ~15);
+            page[b] = cache + (long)tab[j0 / page_size] * page_stride;
+            place[b] = j0 % page_size;
+        }
+        floatx4 s[2];
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            s[b] = floatx4{};
+            const bf16_t* krow = page[b] + (size_t)(place[b] + r) * kd;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const int c = 32 * ks + 8 * q4;
+                uint4 kv = *reinterpret_cast<const uint4*>(krow + (c < kd ? c : 0));
+                if (c >= kd) kv = uint4{0, 0, 0, 0};
+                s[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kv), qreg[ks], s[b], 0, 0, 0);
+            }
+        }
+        // element v of s[b]: position kv0 + 16*b + 4*q4 + v, head r
+        float mx = -INFINITY;
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int j = kv0 + 16 * b + 4 * q4 + v;
+                s[b][v] = (j >= lo && j <= p) ? s[b][v] * scale2 : -INFINITY;
+                mx = fmaxf(mx, s[b][v]);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m, mx);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float corr = exp2_fast(m - m_use);
+        float sum = 0.f;
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                s[b][v] = exp2_fast(s[b][v] - m_use);
+                sum += s[b][v];
+            }
+        sum += __shfl_xor(sum, 16, 64);
+        sum += __shfl_xor(sum, 32, 64);
+        l = l * corr + sum;
+        m = m_new;
+        const uint4 pb = {f32x2_to_bf16x2(s[0][0], s[0][1]), f32x2_to_bf16x2(s[0][2], s[0][3]), f32x2_to_bf16x2(s[1][0], s[1][1]), f32x2_to_bf16x2(s[1][2], s[1][3])};
+        // a block whose positions are all masked was read from another block's place: its probabilities are zeros, which is all that matters
+#pragma unroll
+        for (int i = 0; i < DT; ++i) {
+            const int c = 16 * i + r;
+            const size_t ch = (size_t)(c < vd ? c : 0) * page_size;
+            uint2 v0 = *reinterpret_cast<const uint2*>(page[0] + v_plane + ch + place[0] + 4 * q4);
+            uint2 v1 = *reinterpret_cast<const uint2*>(page[1] + v_plane + ch + place[1] + 4 * q4);
+            if (c >= vd) v0 = v1 = uint2{0, 0};
+#pragma unroll
+            for (int v = 0; v < 4; ++v) o[i][v] *= corr;
+            o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(uint4{v0.x, v0.y, v1.x, v1.y}), as_bf16x8(pb), o[i], 0, 0, 0);
+        }
+    }
+    // element v of o[i]: channel 16*i + 4*q4 + v, head r
+    if (!head_ok) return;
+    if (n_splits == 1) {
+        const float inv = 1.0f / l;                      // (a row always sees itself: l > 0)
+#pragma unroll
+        for (int i = 0; i < DT; ++i)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int c = 16 * i + 4 * q4 + v;
+                if (c < vd) out[((size_t)t * n_heads + head) * vd + c] = f32_to_bf16(o[i][v] * inv);
+            }
+        return;
+    }
+    float* mine = part + (((size_t)t * n_heads + head) * n_splits + sp) * (vd + 2);
+    if (q4 == 0) { mine[0] = m; mine[1] = l; }
+#pragma unroll
+    for (int i = 0; i < DT; ++i)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int c = 16 * i + 4 * q4 + v;
+            if (c < vd) mine[2 + c] = o[i][v];
+        }
+}
+
+// The shares of one (row, head), in their order: out = sum_s 2^(m_s - m) o_s / sum_s 2^(m_s - m) l_s.
+__global__ __launch_bounds__(64) void latent_merge_kernel(const float* __restrict__ part, bf16_t* __restrict__ out, int vd, int n_splits) {
+    const size_t rh = blockIdx.x;
+    const float* mine = part + rh * n_splits * (vd + 2);
+    float m = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) m = fmaxf(m, mine[(size_t)s * (vd + 2)]);
+    float l = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+        const float ms = mine[(size_t)s * (vd + 2)];
+        if (ms != -INFINITY) l += exp2_fast(ms - m) * mine[(size_t)s * (vd + 2) + 1];
+    }
+    for (int c = threadIdx.x; c < vd; c += 64) {
+        float acc = 0.f;
+        for (int s = 0; s < n_splits; ++s) {
+            const float ms = mine[(size_t)s * (vd + 2)];
+            if (ms != -INFINITY) acc = fmaf(exp2_fast(ms - m), mine[(size_t)s * (vd + 2) + 2 + c], acc);
+        }
+        out[rh * vd + c] = f32_to_bf16(acc / l);
+    }
+}
+
 }  // namespace
 
 // proj: float32 [n_rows, ld] = [query latent (q_rank) | key/value latent (kv_rank) | rotated key part (rot)]; cos, sin: float32
-// [n_rows, rot/2]; cq: [n_rows, ldcq] gets the normed query latent; the cache's pages hold [place][kv_rank + rot].
+// [n_rows, rot/2]; cq: [n_rows, ldcq] gets the normed query latent; the cache's pages hold [place][kv_rank + rot], then [kv_rank][place].
 GI_API int gi_latent_prepare(const float* proj, long ld, int q_rank, int kv_rank, int rot, const void* q_norm, const void* kv_norm, int norm_dtype,
                              float eps, const float* cos_t, const float* sin_t, const int* pos, const int* slot, const int* table, int table_stride,
                              void* cq, int cq_dtype, long ldcq, void* cache, int cache_dtype, long page_stride, int page_size, int n_rows,
                              hipStream_t stream) {
     GI_REQUIRE(n_rows > 0 && q_rank > 0 && kv_rank > 0 && rot >= 0 && rot % 2 == 0, "latent_prepare: bad sizes (rows %d, latents %d and %d, %d rotated channels)",
                n_rows, q_rank, kv_rank, rot);
-    GI_REQUIRE(ld >= (long)q_rank + kv_rank + rot && ldcq >= q_rank && page_size > 0 && page_stride >= (long)page_size * (kv_rank + rot),
+    GI_REQUIRE(ld >= (long)q_rank + kv_rank + rot && ldcq >= q_rank && page_size > 0 && page_stride >= (long)page_size * (2L * kv_rank + rot),
                "latent_prepare: rows or pages too small for these latents");
     GI_REQUIRE(rot == 0 || (cos_t != nullptr && sin_t != nullptr), "latent_prepare: a rotation needs its cosines and sines");
     dim3 grid(n_rows, 2);
@@ -107,5 +305,60 @@ GI_API int gi_latent_queries(const float* q, long ldq, const float* cos_t, const
     else return gi_fail("latent_queries: dtypes (%d, %d) are not served", plain_dtype, folded_dtype);
 #undef GO
     GI_CHECK_LAUNCH("latent_queries");
+    return 0;
+}
+
+// a: bfloat16 [n_rows, lda], head h's operand in columns [h*k_dim, (h+1)*k_dim); w: bfloat16 [n_heads][n_out][k_dim]; out: [n_rows, ldo],
+// head h's result in columns [h*out_head_stride, h*out_head_stride + n_out).
+GI_API int gi_heads_product_supports(int k_dim, int n_out) { return k_dim > 0 && n_out > 0 && k_dim % 8 == 0; }
+
+GI_API int gi_heads_product(const void* a, long lda, const void* w, void* out, int out_dtype, long ldo, long out_head_stride, int n_rows, int n_heads, int k_dim,
+                            int n_out, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && n_heads > 0 && n_heads <= 65535 && gi_heads_product_supports(k_dim, n_out), "heads_product: bad sizes (rows %d, heads %d, k %d, n %d; k a multiple of 8)",
+               n_rows, n_heads, k_dim, n_out);
+    GI_REQUIRE(lda % 8 == 0 && lda >= (long)n_heads * k_dim && ((uintptr_t)a & 15) == 0 && ((uintptr_t)w & 15) == 0 && out_head_stride >= n_out &&
+               ldo >= (long)(n_heads - 1) * out_head_stride + n_out, "heads_product: operands must be 16-byte aligned with row strides that are multiples of 8, and rows long enough");
+    GI_REQUIRE((n_out + 63) / 64 <= 65535, "heads_product: too many columns");
+    dim3 grid((n_rows + 15) / 16, n_heads, (n_out + 63) / 64);
+    if (out_dtype == GI_F32) heads_product_kernel<float><<<grid, 64, 0, stream>>>((const bf16_t*)a, lda, (const bf16_t*)w, (float*)out, ldo, out_head_stride, n_rows, k_dim, n_out);
+    else if (out_dtype == GI_BF16) heads_product_kernel<bf16_t><<<grid, 64, 0, stream>>>((const bf16_t*)a, lda, (const bf16_t*)w, (bf16_t*)out, ldo, out_head_stride, n_rows, k_dim, n_out);
+    else return gi_fail("heads_product: unknown output dtype %d", out_dtype);
+    GI_CHECK_LAUNCH("heads_product");
+    return 0;
+}
+
+// Sizes the matrix-core latent attention takes: keys of up to 288 channels in 16-byte pieces, values of up to 256 channels, pages of whole blocks of 16 places.
+GI_API int gi_latent_attention_supports(int kd, int vd, int page_size) {
+    return kd > 0 && kd % 8 == 0 && kd <= 288 && vd > 0 && vd <= 256 && vd <= kd && page_size > 0 && page_size % 16 == 0;
+}
+GI_API long gi_latent_attention_scratch_floats(int n_rows, int n_heads, int vd, int n_splits) {
+    return n_splits > 1 ? (long)n_rows * n_heads * n_splits * (vd + 2) : 0;
+}
+
+// q: bfloat16 [n_rows, n_heads*kd] (folded queries); cache: bfloat16 pages [place][kd] then [vd][place]; out: bfloat16 [n_rows, n_heads*vd].
+GI_API int gi_latent_attention_bf16(const void* q, const void* cache, void* out, float* part, long part_floats, const int* pos, const int* slot, const int* table,
+                                    int table_stride, long page_stride, int page_size, int n_rows, int n_heads, int kd, int vd, int window, float scale,
+                                    int n_splits, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && n_heads > 0 && gi_latent_attention_supports(kd, vd, page_size), "latent_attention: sizes (rows %d, heads %d, keys %d, values %d, pages of %d) are not taken",
+               n_rows, n_heads, kd, vd, page_size);
+    GI_REQUIRE(window >= 0 && n_splits >= 1 && n_splits <= 64 && page_stride >= (long)page_size * (kd + vd) && page_stride % 8 == 0 && ((uintptr_t)cache & 15) == 0 &&
+               ((uintptr_t)q & 15) == 0, "latent_attention: bad window, shares, page stride or alignment");
+    GI_REQUIRE(part_floats >= gi_latent_attention_scratch_floats(n_rows, n_heads, vd, n_splits) && (n_splits == 1 || part != nullptr), "latent_attention: scratch of %ld floats needed, %ld given",
+               gi_latent_attention_scratch_floats(n_rows, n_heads, vd, n_splits), part_floats);
+    GI_REQUIRE((long)n_rows * n_heads < 2147483647L && (n_heads + 15) / 16 <= 65535, "latent_attention: too many rows or heads");
+    dim3 grid(n_rows, (n_heads + 15) / 16, n_splits);
+    const float scale2 = scale * 1.4426950408889634f;
+#define GO(KS, DT)                                                                                                                                      \
+    latent_attention_kernel<KS, DT><<<grid, 64, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, (bf16_t*)out, part, pos, slot, table, table_stride, \
+                                                             page_stride, page_size, n_heads, kd, vd, window, scale2, n_splits)
+    if (kd <= 96 && vd <= 64) GO(3, 4);
+    else if (kd <= 160 && vd <= 128) GO(5, 8);
+    else GO(9, 16);
+#undef GO
+    GI_CHECK_LAUNCH("latent_attention");
+    if (n_splits > 1) {
+        latent_merge_kernel<<<(unsigned)(n_rows * n_heads), 64, 0, stream>>>(part, (bf16_t*)out, vd, n_splits);
+        GI_CHECK_LAUNCH("latent_merge");
+    }
     return 0;
 }

@@ -311,19 +311,25 @@ __global__ __launch_bounds__(256) void delta_tail_kernel(const float* __restrict
 }
 
 // The rule itself: one wave per (request of the step, head, four columns of S).  lane = column * 16 + group of rows; a lane keeps
-// the rows 16 apart of its column.  State of a request slot: [head][tile]{[dk][4]}.  Key and query of a block of tokens wait in
-// LDS; every sum over the key's rows is the lanes' own shares in a fixed order, then the 16 groups by lane moves.
+// the rows 16 apart of its column.  State of a request slot: [head][tile]{[dk][4]}.
+// With S the memory before the token, S' = g S + k w^T after it and w = beta (v - g S^T k), the read-out is
+//     o = S'^T q = g S^T q + w (k . q):
+// both sums over the old memory's rows (S^T k and S^T q) and k . q are taken in one pass and reduced side by side, the memory is
+// updated behind them, and a token's chain of dependent steps is one pass and one reduction, not two of each.  Every sum over the
+// key's rows is the lanes' own shares in a fixed order, then the 16 groups by lane moves: the bits do not depend on the cut.
+// Key and query of a block of tokens wait in LDS; the block after it is asked for while this one is worked on.
 template <int ROWS>
 __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict__ qkv, long ld, const float* __restrict__ gates,
                                                        const int* __restrict__ seg_start, const int* __restrict__ seg_len,
                                                        const int* __restrict__ row_slot, float* __restrict__ state, long state_stride,
                                                        float* __restrict__ out, long ldo, int n_heads, int n_kv, int dk, int dv) {
     constexpr int C = 4, RG = 16, KQ = RG * ROWS;
-    constexpr int TB = (2048 / KQ) < 16 ? (2048 / KQ) : 16;      // tokens staged at a time
-    static_assert(TB >= 4, "a block of at least four tokens fits");
-    __shared__ float2 kq_s[TB][KQ];
-    __shared__ float v_s[TB][C];
-    __shared__ float2 gb_s[TB];
+    constexpr int TB = (1024 / KQ) < 16 ? (1024 / KQ) : 16;      // tokens staged at a time
+    constexpr int PER = TB * KQ / 64;            // (k, q) pairs a lane brings per block
+    static_assert(TB >= 2 && TB * C <= 64, "a block of 2 to 16 tokens; a lane brings one value and one pair of gates");
+    __shared__ float2 kq_s[2][TB][KQ];
+    __shared__ float v_s[2][TB][C];
+    __shared__ float2 gb_s[2][TB];
     const int seg = blockIdx.x, h = blockIdx.y, vt = blockIdx.z, n_tiles = gridDim.z;
     const int lane = threadIdx.x, c = lane / RG, rg = lane % RG;
     const int n = seg_len[seg];
@@ -340,40 +346,62 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict_
         const int i = rr * RG + rg;
         S[rr] = i < dk ? st[(size_t)i * C + c] : 0.f;
     }
-    for (int b0 = 0; b0 < n; b0 += TB) {
-        const int here = min(TB, n - b0);
-        __syncthreads();                                          // the block before has been read
-        for (int idx = lane; idx < here * KQ; idx += 64) {
-            const int u = idx / KQ, i = idx % KQ;
-            const float* row = qkv + (size_t)(t0 + b0 + u) * ld;
-            kq_s[u][i] = i < dk ? float2{row[k_at + i], row[q_at + i]} : float2{0.f, 0.f};
-        }
-        if (lane < here * C) {
-            const int u = lane / C, cc = vt * C + lane % C;
-            v_s[u][lane % C] = cc < dv ? qkv[(size_t)(t0 + b0 + u) * ld + v_at + cc] : 0.f;
-        }
-        if (lane < here) {
-            const float* g = gates + (size_t)(t0 + b0 + lane) * 2 * n_heads;
-            gb_s[lane] = float2{g[h], g[n_heads + h]};
-        }
-        __syncthreads();
-        for (int u = 0; u < here; ++u) {
-            const float2 gb = gb_s[u];
-            float held = 0.f;
+    // A block of TB tokens from `first` on (rows beyond the request's last are read as its last: finite, and never used).
+    float2 kq_reg[PER], gb_reg;
+    float v_reg;
+    auto fetch = [&](int first) {
 #pragma unroll
-            for (int rr = 0; rr < ROWS; ++rr) held = fmaf(S[rr], kq_s[u][rr * RG + rg].x, held);
-            held = gb.x * group_sum<RG>(held);                    // what the decayed memory holds along the key
-            const float w = gb.y * (v_s[u][c] - held);
-            float acc = 0.f;
+        for (int e = 0; e < PER; ++e) {
+            const int idx = lane + 64 * e, u = idx / KQ, i = idx % KQ;
+            const float* row = qkv + (size_t)(t0 + min(first + u, n - 1)) * ld;
+            const int ic = min(i, dk - 1);
+            const float kk = row[k_at + ic], qq = row[q_at + ic];
+            kq_reg[e] = i < dk ? float2{kk, qq} : float2{0.f, 0.f};
+        }
+        const int u = min(lane / C, TB - 1), cc = min(vt * C + lane % C, dv - 1);
+        v_reg = qkv[(size_t)(t0 + min(first + u, n - 1)) * ld + v_at + cc];
+        const float* g = gates + (size_t)(t0 + min(first + min(lane, TB - 1), n - 1)) * 2 * n_heads;
+        gb_reg = float2{g[h], g[n_heads + h]};
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int e = 0; e < PER; ++e) {
+            const int idx = lane + 64 * e;
+            kq_s[buf][idx / KQ][idx % KQ] = kq_reg[e];
+        }
+        if (lane < TB * C) v_s[buf][lane / C][lane % C] = v_reg;
+        if (lane < TB) gb_s[buf][lane] = gb_reg;
+    };
+    fetch(0);
+    stash(0);
+    barrier_lds();
+    int buf = 0;
+    for (int b0 = 0; b0 < n; b0 += TB, buf ^= 1) {
+        const int here = min(TB, n - b0);
+        const bool more = b0 + TB < n;
+        if (more) fetch(b0 + TB);
+        for (int u = 0; u < here; ++u) {
+            const float2 gb = gb_s[buf][u];
+            float kx[ROWS];
+            float sk = 0.f, sq = 0.f, kq = 0.f;
 #pragma unroll
             for (int rr = 0; rr < ROWS; ++rr) {
-                const float2 kq = kq_s[u][rr * RG + rg];
-                S[rr] = fmaf(gb.x, S[rr], kq.x * w);
-                acc = fmaf(S[rr], kq.y, acc);
+                const float2 pair = kq_s[buf][u][rr * RG + rg];
+                kx[rr] = pair.x;
+                sk = fmaf(S[rr], pair.x, sk);
+                sq = fmaf(S[rr], pair.y, sq);
+                kq = fmaf(pair.x, pair.y, kq);
             }
-            acc = group_sum<RG>(acc);
-            if (rg == 0 && live) out[(size_t)(t0 + b0 + u) * ldo + h * dv + col] = acc;
+            sk = group_sum<RG>(sk);
+            sq = group_sum<RG>(sq);
+            kq = group_sum<RG>(kq);
+            const float w = gb.y * (v_s[buf][u][c] - gb.x * sk);       // beta (v - g S^T k)
+#pragma unroll
+            for (int rr = 0; rr < ROWS; ++rr) S[rr] = fmaf(gb.x, S[rr], kx[rr] * w);
+            if (rg == 0 && live) out[(size_t)(t0 + b0 + u) * ldo + h * dv + col] = fmaf(gb.x, sq, w * kq);
         }
+        if (more) stash(buf ^ 1);                // (the buffer the block before this one was read from)
+        barrier_lds();
     }
 #pragma unroll
     for (int rr = 0; rr < ROWS; ++rr) {

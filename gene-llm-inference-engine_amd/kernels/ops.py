@@ -35,7 +35,7 @@ _SIGNATURES = {
     "gi_softcap_rows": [c_void_p, c_int, c_int, c_long, c_float, c_void_p],
     "gi_gemm_exact": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p],
     "gi_attention_exact": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int,
-                           c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_long, c_int, c_void_p],
+                           c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_long, c_void_p],
     "gi_rmsnorm_add": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_long, c_long, c_void_p],
     "gi_rmsnorm_add_norm": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_long, c_long, c_long, c_void_p],
     "gi_norm_rope_store": [c_void_p, c_void_p, c_void_p, c_long, c_long, c_long, c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int,
@@ -48,6 +48,9 @@ _SIGNATURES = {
     "gi_delta_scan": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_long, c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p],
     "gi_latent_prepare": [c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                           c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_int, c_int, c_void_p],
+    "gi_heads_product": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_long, c_long, c_int, c_int, c_int, c_int, c_void_p],
+    "gi_latent_attention_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int,
+                                 c_float, c_int, c_void_p],
     "gi_latent_queries": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gi_act_mul": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "gi_segments": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p],
@@ -109,6 +112,8 @@ def lib():
         l.gi_mlstm_state_floats.restype = c_long
         l.gi_mlstm_max_key_dim.argtypes = []
         l.gi_mlstm_max_key_dim.restype = c_int
+        l.gi_latent_attention_supports.argtypes = [c_int, c_int, c_int]
+        l.gi_latent_attention_supports.restype = c_int
         l.gi_probe_mfma_flops.argtypes = [c_int, c_int]
         l.gi_probe_mfma_flops.restype = c_long
         _lib = l
@@ -429,12 +434,11 @@ def _check_paged(cache, table, what):
 
 
 def attention_exact(q, cache, out, positions, slots, table, n_heads, n_kv, hd, window=None, scale=None, *, page_size=None, value_dim=None,
-                    chunk=None, sinks=None, gate=None, values_in_keys=False):
+                    chunk=None, sinks=None, gate=None):
     """Each row attends over its request's cached keys up to its own position, no further back than `window` positions and not
     beyond the start of its own chunk of `chunk` positions.  value_dim: channels of a value head (hd if not given); sinks:
     float32 [heads], a score per head that joins the softmax's denominator only; gate: float32 [n, >= heads] (unit inner
-    stride), head h's output is multiplied by sigmoid(gate[t, h]).  values_in_keys: the pages hold keys only, and a position's value is
-    the first value_dim channels of its key."""
+    stride), head h's output is multiplied by sigmoid(gate[t, h])."""
     _dev(q, cache, out, positions, slots, table, sinks, gate)
     n = q.shape[0]
     vd = int(value_dim or hd)
@@ -454,7 +458,7 @@ def attention_exact(q, cache, out, positions, slots, table, n_heads, n_kv, hd, w
     _call("gi_attention_exact", q.data_ptr(), _code(q, "attention: q"), cache.data_ptr(), _code(cache, "attention: cache"), out.data_ptr(),
           _code(out, "attention: out"), positions.data_ptr(), slots.data_ptr(), table.data_ptr(), table.stride(0), cache.stride(0),
           page_size, n, n_heads, n_kv, hd, vd, int(window or 0), int(chunk or 0), float(scale if scale is not None else hd ** -0.5),
-          _ptr(sinks), _ptr(gate), gate.stride(0) if gate is not None else 0, 1 if values_in_keys else 0, _stream())
+          _ptr(sinks), _ptr(gate), gate.stride(0) if gate is not None else 0, _stream())
     return out
 
 
@@ -740,7 +744,8 @@ def delta_scan(qkv, gates, seg_start, seg_len, row_slot, state, out, n_heads, n_
 def latent_prepare(proj, q_rank, kv_rank, rot, q_norm, kv_norm, eps, cos, sin, positions, slots, table, cq, cache, page_size):
     """proj float32 [n, q_rank + kv_rank + rot]: the query latent, RMS-normed with q_norm, into cq [n, q_rank]; the key/value latent,
     RMS-normed with kv_norm, and the last rot channels turned in neighbouring pairs (cos, sin float32 [n, rot/2]), into the row's
-    place of its page, [place][kv_rank + rot]."""
+    place of its page: the keys [place][kv_rank + rot], and the latent once more behind them with the places innermost, [kv_rank][place]
+    (a layer of one key/value head with keys of kv_rank + rot and values of kv_rank channels)."""
     _dev(proj, q_norm, kv_norm, cos, sin, positions, slots, table, cq, cache)
     n = proj.shape[0]
     if not (proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= q_rank + kv_rank + rot):
@@ -754,7 +759,7 @@ def latent_prepare(proj, q_rank, kv_rank, rot, q_norm, kv_norm, eps, cos, sin, p
             if not (t.dtype == torch.float32 and t.shape == (n, rot // 2) and t.is_contiguous()):
                 raise KernelError("latent_prepare: cos/sin must be float32 [n, rot/2]")
     _check_paged(cache, table, "latent_prepare")
-    if cache.stride(0) < page_size * (kv_rank + rot):
+    if cache.stride(0) < page_size * (2 * kv_rank + rot):
         raise KernelError("latent_prepare: the pages are too small for these latents")
     _i32(positions, "latent_prepare: positions", n)
     _i32(slots, "latent_prepare: slots", n)
@@ -1055,18 +1060,17 @@ def attention(q, cache, out, ctx, table, n_heads, n_kv, hd, window=None):
     return attention_exact(q, cache, out, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window)
 
 
-def attention_general(q, cache, out, ctx, table, n_heads, n_kv, hd, *, page_size, value_dim=None, window=None, chunk=None, scale=None, sinks=None, gate=None,
-                      values_in_keys=False):
+def attention_general(q, cache, out, ctx, table, n_heads, n_kv, hd, *, page_size, value_dim=None, window=None, chunk=None, scale=None, sinks=None, gate=None):
     """Attention of a step's rows for layers with any of: value heads of another size, a scale of their own, a mask cut into
-    chunks, sinks, a gate per head, values that are the first channels of the keys."""
+    chunks, sinks, a gate per head."""
     vd = int(value_dim or hd)
-    if (vd == hd and not values_in_keys and cache.dim() == 5 and q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
+    if (vd == hd and cache.dim() == 5 and q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
             and (gate is None or gate.dtype == torch.float32)):
         plan = _plan_of(ctx)
         if (not plan.n_tiles or attention_bf16_supports(hd, page_size, True)) and (not plan.n_decode or attention_bf16_supports(hd, page_size, False)):
             return attention_bf16(q, cache, out, plan, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window, scale, chunk=chunk, sinks=sinks, gate=gate)
     return attention_exact(q, cache, out, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window, scale, page_size=page_size,
-                           value_dim=value_dim, chunk=chunk, sinks=sinks, gate=gate, values_in_keys=values_in_keys)
+                           value_dim=value_dim, chunk=chunk, sinks=sinks, gate=gate)
 
 
 # Up to so many rows the decode kernel rotates and writes the pages itself.  It saves the rotation kernel's launch wherever the
@@ -1313,3 +1317,50 @@ def measured_mfma_rate(device="cuda:0", iters: int = 20000, repeats: int = 5) ->
     sink = torch.empty(n_blocks * 256, dtype=torch.float32, device=device)
     ms = _timed_ms(lambda: _call("gi_probe_mfma", iters, sink.data_ptr(), n_blocks, _stream()), repeats)
     return lib().gi_probe_mfma_flops(iters, n_blocks) / (ms * 1e-3) / 1e12
+
+
+def heads_product(a, w, out, n_heads, out_head_stride=None):
+    """out[t, h*stride + n] = sum_k a[t, h*k_dim + k] * w[h, n, k] for every head in one launch, on the matrix cores: a bfloat16
+    [rows, heads*k_dim], w bfloat16 [heads, n_out, k_dim] contiguous, out [rows, >= heads*stride] bfloat16 or float32 (stride: n_out
+    if not given).  False, and nothing done, where the kernel does not take the operands (the caller then multiplies head by head)."""
+    _dev(a, w, out)
+    rows, k_dim, n_out = a.shape[0], w.shape[2], w.shape[1]
+    stride = int(out_head_stride or n_out)
+    if not (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.is_contiguous() and w.shape[0] == n_heads and a.shape[1] == n_heads * k_dim and a.stride(1) == 1
+            and out.stride(1) == 1 and out.dtype in (torch.bfloat16, torch.float32) and k_dim % 8 == 0 and a.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+            and out.shape[0] == rows and out.shape[1] >= (n_heads - 1) * stride + n_out):
+        return False
+    if _profile is not None:
+        _profile.note = (f"{n_heads}x{n_out}x{k_dim}", w.numel() * w.element_size())
+    _call("gi_heads_product", a.data_ptr(), a.stride(0), w.data_ptr(), out.data_ptr(), _code(out, "heads_product: out"), out.stride(0), stride, rows, n_heads, k_dim, n_out, _stream())
+    return True
+
+
+@lru_cache(maxsize=None)
+def latent_attention_bf16_supports(kd, vd, page_size) -> bool:
+    return bool(lib().gi_latent_attention_supports(kd, vd, page_size))
+
+
+def latent_attention_bf16(q, cache, out, ctx, table, n_heads, kd, vd, page_size, window=None, scale=1.0):
+    """Attention of a step's rows over latent pages (one key/value head for all query heads: keys [place][kd], then the values
+    [vd][place]) on the matrix cores; q bfloat16 [n, heads*kd], out bfloat16 [n, heads*vd].  Every row is a wave per 16 heads and
+    share of its context; with few rows the context is shared out further and a second kernel adds the shares."""
+    _dev(q, cache, out, table)
+    n = q.shape[0]
+    if not (q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and q.shape == (n, n_heads * kd) and q.is_contiguous()
+            and out.shape == (n, n_heads * vd) and out.is_contiguous()):
+        raise KernelError("latent_attention: q must be bfloat16 [n, heads*kd] and out bfloat16 [n, heads*vd], contiguous, over a bfloat16 cache")
+    _check_paged(cache, table, "latent_attention")
+    _i32(ctx.row_pos, "latent_attention: positions", n)
+    _i32(ctx.row_slot, "latent_attention: slots", n)
+    plan = _plan_of(ctx)                  # (its longest context is the bracket's in a captured pass: the same for every replay)
+    span = max(plan.max_decode_context, plan.max_tile_context, 1)
+    if window:
+        span = min(span, int(window) + 31)
+    groups = n * (-(-n_heads // 16))
+    n_splits = max(1, min(16, 2048 // groups, (span + 63) // 64))
+    n_part = n * n_heads * n_splits * (vd + 2) if n_splits > 1 else 0
+    part = torch.empty(n_part, dtype=torch.float32, device=out.device) if n_part else None
+    _call("gi_latent_attention_bf16", q.data_ptr(), cache.data_ptr(), out.data_ptr(), _ptr(part), n_part, ctx.row_pos.data_ptr(), ctx.row_slot.data_ptr(), table.data_ptr(),
+          table.stride(0), cache.stride(0), int(page_size), n, n_heads, kd, vd, int(window or 0), float(scale), n_splits, _stream())
+    return out

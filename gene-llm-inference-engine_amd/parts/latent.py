@@ -4,13 +4,16 @@
 What is cached per position is the normed key/value latent c [kv_rank] and one rotated key part [rotary_dim], nothing per
 head.  The up projections are folded into the two sides of the attention instead of being applied to cached rows:
     score_j = (W_uk_h^T q_plain_h) . c_j + q_rot_h . k_rot_j        o_h = W_uv_h (sum_j p_j c_j)
-so the attention kernel sees one key/value head of kv_rank + rotary_dim channels whose first kv_rank channels are also the
-value, shared by all query heads, and every step costs the same few products whatever the context holds.
+so the attention kernel sees one key/value head, shared by all query heads, with keys [c; k_rot] of kv_rank + rotary_dim
+channels and values c of kv_rank channels, and every step costs the same few products whatever the context holds.  The pages
+are those of any layer whose values are shorter than its keys (the latent lies in them twice: as part of the key, and as the
+value with the places innermost, which is how the kernels' second product reads it).
 
 Steps of a pass: one product with [W_dq; W_dkv]; one kernel that norms both latents, turns the rotated key part and writes the
-page; the product with W_uq; one kernel that parts every head's query into plain channels (rows for the folding products) and
-turned channels (written where the attention reads them); per head the folding product with W_uk_h^T; attention; per head the
-product with W_uv_h; the output product onto the residual."""
+page; the product with W_uq; one kernel that parts every head's query into plain channels (rows for the folding product) and
+turned channels (written where the attention reads them); the folding product with every head's W_uk_h^T; attention (in
+bfloat16 on the matrix cores: 16 heads are the columns of one matrix instruction, for a single decoded row too); the product
+with every head's W_uv_h; the output product onto the residual."""
 from __future__ import annotations
 
 import torch
@@ -29,6 +32,17 @@ def _head_product(a, w, out):
     if out.data_ptr() % 16 or (out.stride(0) * out.element_size()) % 16 or a.data_ptr() % 16:
         return ops.gemm_exact(a, w, out)
     return linear(a, w, out)
+
+
+def heads_product(a, w, out, n_heads, out_head_stride=None):
+    """out[:, h*stride : h*stride + n] = a[:, h*k : (h+1)*k] @ w[h].T for every head: one launch in bfloat16, head by head otherwise."""
+    k, n = w.shape[2], w.shape[1]
+    stride = out_head_stride or n
+    if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and ops.heads_product(a, w, out, n_heads, stride):
+        return out
+    for i in range(n_heads):
+        _head_product(a[:, i * k:(i + 1) * k], w[i], out[:, i * stride:i * stride + n])
+    return out
 
 
 class LatentAttention(Mixer):
@@ -55,7 +69,7 @@ class LatentAttention(Mixer):
         self.w_uq = tensors[s.uq_proj]
         # per head: W_uk_h^T [kv_rank, head_dim] (folded into the queries) and W_uv_h [value_dim, kv_rank] (applied to the attended latent)
         self.w_uk_t = tensors[s.uk_proj].view(s.n_heads, s.head_dim, s.kv_rank).transpose(1, 2).contiguous()
-        self.w_uv = tensors[s.uv_proj].view(s.n_heads, s.value_dim, s.kv_rank)
+        self.w_uv = tensors[s.uv_proj].view(s.n_heads, s.value_dim, s.kv_rank).contiguous()
         self.w_o = tensors[s.o_proj]
         self.in_dtype = activation_dtype_for(self.w_down, dtype)
         self.cq_dtype = activation_dtype_for(self.w_uq, dtype)
@@ -76,7 +90,7 @@ class LatentAttention(Mixer):
 
     @classmethod
     def cache_need(cls, spec):
-        return PagedKvNeed(1, spec.kv_rank + spec.rotary_dim, spec.window, spec.kv_rank, None, values_in_keys=True)
+        return PagedKvNeed(1, spec.kv_rank + spec.rotary_dim, spec.window, spec.kv_rank, None)
 
     def forward(self, h, residual, ctx, cache, overwrite=False):
         s, T, dev = self.spec, ctx.n_rows, ctx.device
@@ -92,16 +106,17 @@ class LatentAttention(Mixer):
         plain = torch.empty((T, H * s.head_dim), dtype=self.plain_dtype, device=dev)
         folded = torch.empty((T, H * kd), dtype=cache.kv.dtype, device=dev)
         ops.latent_queries(q, cos, sin, plain, folded, H, s.head_dim, s.rotary_dim, s.kv_rank)
-        for i in range(H):
-            _head_product(plain[:, i * s.head_dim:(i + 1) * s.head_dim], self.w_uk_t[i], folded[:, i * kd:i * kd + s.kv_rank])
+        heads_product(plain, self.w_uk_t, folded, H, kd)
         attended = torch.empty((T, H * s.kv_rank), dtype=cache.kv.dtype, device=dev)
-        ops.attention_general(folded, cache.kv, attended, ctx, cache.table, H, 1, kd, page_size=cache.page_size, value_dim=s.kv_rank,
-                              window=s.window, scale=s.scale, values_in_keys=True)
+        if cache.kv.dtype == torch.bfloat16 and ops.latent_attention_bf16_supports(kd, s.kv_rank, cache.page_size):
+            ops.latent_attention_bf16(folded, cache.kv, attended, ctx, cache.table, H, kd, s.kv_rank, cache.page_size, s.window, s.scale)
+        else:
+            ops.attention_general(folded, cache.kv, attended, ctx, cache.table, H, 1, kd, page_size=cache.page_size, value_dim=s.kv_rank,
+                                  window=s.window, scale=s.scale)
         if attended.dtype != activation_dtype_for(self.w_uv, self.dtype):
             attended = attended.to(activation_dtype_for(self.w_uv, self.dtype))
         att = torch.empty((T, H * s.value_dim), dtype=self.att_dtype, device=dev)
-        for i in range(H):
-            _head_product(attended[:, i * s.kv_rank:(i + 1) * s.kv_rank], self.w_uv[i], att[:, i * s.value_dim:(i + 1) * s.value_dim])
+        heads_product(attended, self.w_uv, att, H)
         if overwrite:
             linear(att, self.w_o, residual)
         else:

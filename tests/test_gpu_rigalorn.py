@@ -222,8 +222,8 @@ def test_attention_with_biases_blended_values_and_one_key_that_stands_out(T, win
 
 @pytest.mark.parametrize("T, window, far", [(200, None, 2), (200, 50, 150), (200, 50, 149), (45, 16, 29), (45, 16, 30)])
 def test_attention_through_latents_against_keys_and_values_made_in_full(T, window, far):
-    """The kernels around the latent cache and the attention whose values are the keys' first channels, with the up projections
-    folded into query and output by hand here, against the plain layer that makes every head's keys and values of every position."""
+    """The kernels around the latent cache and the attention over it, with the up projections folded into query and output by hand
+    here, against the plain layer that makes every head's keys and values of every position."""
     from geneinfer_amd.kernels import ops
     H, d, r, dv, q_rank, rank, page, scale, eps = 3, 12, 6, 7, 20, 18, 4, 0.3, 1e-5
     g = torch.Generator().manual_seed(T + far)
@@ -237,7 +237,7 @@ def test_attention_through_latents_against_keys_and_values_made_in_full(T, windo
     want = P.latent_attention(h.double(), {k: v.double() for k, v in w.items()}, m, eps)
 
     dev = lambda t: t.to(DEV)
-    cache, table = _paged(T, page, rank + r, torch.float32, seed=far)
+    cache, table = _paged(T, page, 2 * rank + r, torch.float32, seed=far)
     ctx = _ctx(T)
     f, _ = P.rotary_frequencies(r, 40.0)
     cos, sin = torch.empty(T, r // 2, device=DEV), torch.empty(T, r // 2, device=DEV)
@@ -251,9 +251,82 @@ def test_attention_through_latents_against_keys_and_values_made_in_full(T, windo
     uk = dev(w["uk"]).view(H, d, rank)
     folded.view(T, H, rank + r)[:, :, :rank] = torch.einsum("thd,hdr->thr", plain_part.view(T, H, d), uk)
     att = torch.empty(T, H * rank, device=DEV)
-    ops.attention_general(folded, cache, att, ctx, table, H, 1, rank + r, page_size=page, value_dim=rank, window=window, scale=scale, values_in_keys=True)
+    ops.attention_general(folded, cache, att, ctx, table, H, 1, rank + r, page_size=page, value_dim=rank, window=window, scale=scale)
     got = torch.einsum("thr,hvr->thv", att.view(T, H, rank), dev(w["uv"]).view(H, dv, rank)).reshape(T, H * dv)
     assert relative_error(got, want) < 3e-5
+
+
+@pytest.mark.parametrize("H, kd, vd, window, lens, pos0", [(20, 144, 128, 40, [1, 1, 1], [700, 39, 0]), (8, 80, 64, None, [130, 1], [0, 300]), (32, 288, 256, 100, [70], [50]),
+                                                          (3, 24, 16, 17, [33, 2, 1], [15, 16, 17]), (16, 96, 64, 1, [20], [0])])
+def test_matrix_core_attention_over_latent_pages(H, kd, vd, window, lens, pos0):
+    """Requests at other positions each, on shuffled pages: single rows whose context is shared out over several waves, and
+    portions of prompts; heads that fill one and a half matrix instructions; keys that are no multiple of 32 channels.  One key
+    just inside every row's window stands out."""
+    from geneinfer_amd.kernels import ops
+    from geneinfer_amd.parts import StepContext
+    g = torch.Generator().manual_seed(H + kd)
+    page, scale = 16, 0.2
+    total = [p + n for p, n in zip(pos0, lens)]
+    n_pages = sum(-(-t // page) for t in total)
+    order = torch.randperm(n_pages + 2, generator=g).tolist()
+    table = torch.full((len(lens) + 1, max(-(-t // page) for t in total) + 1), -1, dtype=torch.int32)
+    cache = torch.zeros(n_pages + 2, page * (kd + vd), dtype=torch.bfloat16)
+    keys = []
+    for s, t in enumerate(total):
+        k = torch.randn(t, kd, generator=g).to(torch.bfloat16)
+        keys.append(k)
+        for i in range(-(-t // page)):
+            pg = order.pop()
+            table[s, i] = pg
+            block = k[i * page:(i + 1) * page]
+            cache[pg, :block.shape[0] * kd] = block.reshape(-1)
+            values = torch.zeros(vd, page, dtype=torch.bfloat16)
+            values[:, :block.shape[0]] = block[:, :vd].T
+            cache[pg, page * kd:] = values.reshape(-1)
+    q = torch.randn(sum(lens), H * kd, generator=g)
+    row = 0
+    want = []
+    for s, (p0, n) in enumerate(zip(pos0, lens)):
+        kf = keys[s].double()
+        for i in range(n):
+            p = p0 + i
+            lo = 0 if window is None else max(0, p - window + 1)
+            q.view(-1, H, kd)[row + i, :, :8] = 4.0 * kf[lo, :8] / kf[lo, :8].norm()        # the oldest key the row sees stands out
+        qb = q[row:row + n].to(torch.bfloat16).double().view(n, H, kd)
+        scores = torch.einsum("thd,sd->hts", qb, kf) * scale
+        i_, j_ = torch.arange(p0, p0 + n)[:, None], torch.arange(total[s])[None, :]
+        seen = (j_ <= i_) & ((i_ - j_ < window) if window is not None else True)
+        pr = torch.softmax(scores.masked_fill(~seen[None], float("-inf")), -1)
+        want.append(torch.einsum("hts,sd->thd", pr, kf[:, :vd]).reshape(n, H * vd))
+        row += n
+    want = torch.cat(want)
+    T = sum(lens)
+    starts = [sum(lens[:i]) for i in range(len(lens))]
+    pos = torch.tensor([p + i for p, n in zip(pos0, lens) for i in range(n)], dtype=torch.int32, device=DEV)
+    slots = torch.tensor([s for s, n in enumerate(lens) for _ in range(n)], dtype=torch.int32, device=DEV)
+    ctx = StepContext(n_rows=T, dtype=torch.bfloat16, device=torch.device(DEV), tokens=slots, row_pos=pos, row_slot=slots, seg_slot=list(range(len(lens))),
+                      seg_start=starts, seg_len=list(lens), seg_pos0=list(pos0))
+    assert ops.latent_attention_bf16_supports(kd, vd, page)
+    out = torch.empty(T, H * vd, dtype=torch.bfloat16, device=DEV)
+    ops.latent_attention_bf16(q.to(DEV, torch.bfloat16), cache.to(DEV), out, ctx, table.to(DEV), H, kd, vd, page, window, scale)
+    assert relative_error(out, want) < 1.5e-2                                   # (probabilities and outputs are kept in bfloat16)
+    exact = torch.empty(T, H * vd, dtype=torch.bfloat16, device=DEV)
+    ops.attention_general(q.to(DEV, torch.bfloat16), cache.to(DEV), exact, ctx, table.to(DEV), H, 1, kd, page_size=page, value_dim=vd, window=window, scale=scale)
+    assert relative_error(exact, want) < 6e-3 and relative_error(out, exact.double()) < 1.5e-2
+
+
+@pytest.mark.parametrize("rows, H, k, n", [(1, 8, 32, 128), (37, 3, 72, 40), (300, 32, 64, 256), (16, 2, 256, 64), (5, 1, 8, 7)])
+def test_every_head_s_product_in_one_launch(rows, H, k, n):
+    from geneinfer_amd.kernels import ops
+    g = torch.Generator().manual_seed(rows + k)
+    a, w = torch.randn(rows, H * k, generator=g).to(torch.bfloat16), torch.randn(H, n, k, generator=g).to(torch.bfloat16)
+    want = torch.einsum("thk,hnk->thn", a.double().view(rows, H, k), w.double())
+    for dtype, stride, tol in ((torch.float32, n, 1e-5), (torch.bfloat16, n + 24, 5e-3)):
+        out = torch.zeros(rows, H * stride, dtype=dtype, device=DEV)
+        assert ops.heads_product(a.to(DEV), w.to(DEV), out, H, stride)
+        got = out.view(rows, H, stride)
+        assert relative_error(got[:, :, :n], want) < tol and (got[:, :, n:] == 0).all()
+    assert not ops.heads_product(a.to(DEV)[:, 1:], w.to(DEV), out, H, n)           # operands it does not take: the caller goes head by head
 
 
 # =============================================================================================== whole models

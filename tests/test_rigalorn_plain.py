@@ -193,6 +193,6 @@ def test_cache_needs_by_layer_kind():
     spec = parse_config(CONFIGS["A"]).model_spec()
     needs = [block_class(l.block).cache_need(l) for l in spec.layers]
     assert isinstance(needs[0], StateNeed) and needs[0].shape == (4 * 6 * 16 * 4 + 3 * (2 * 2 * 16 + 4 * 24),)
-    assert needs[1] == PagedKvNeed(1, 40, 20, 32, None, True) and needs[1].elements_per_position() == 40
+    assert needs[1] == PagedKvNeed(1, 40, 20, 32, None) and needs[1].elements_per_position() == 72
     assert needs[2] == PagedKvNeed(2, 32, 12, 16, None) and needs[4] == PagedKvNeed(2, 24, 9, 16, None)
     assert needs[1].first_visible(25) == 6 and needs[2].first_visible(11) == 0 and needs[2].first_visible(12) == 1
