@@ -327,9 +327,9 @@ GI_API int gi_heads_product(const void* a, long lda, const void* w, void* out, i
     return 0;
 }
 
-// Sizes the matrix-core latent attention takes: keys of up to 288 channels in 16-byte pieces, values of up to 256 channels, pages of whole blocks of 16 places.
+// Sizes the matrix-core latent attention takes: keys of up to 576 channels in 16-byte pieces, values of up to 512 channels, pages of whole blocks of 16 places.
 GI_API int gi_latent_attention_supports(int kd, int vd, int page_size) {
-    return kd > 0 && kd % 8 == 0 && kd <= 288 && vd > 0 && vd <= 256 && vd <= kd && page_size > 0 && page_size % 16 == 0;
+    return kd > 0 && kd % 8 == 0 && kd <= 576 && vd > 0 && vd <= 512 && vd <= kd && page_size > 0 && page_size % 16 == 0;
 }
 GI_API long gi_latent_attention_scratch_floats(int n_rows, int n_heads, int vd, int n_splits) {
     return n_splits > 1 ? (long)n_rows * n_heads * n_splits * (vd + 2) : 0;
@@ -353,7 +353,8 @@ GI_API int gi_latent_attention_bf16(const void* q, const void* cache, void* out,
                                                              page_stride, page_size, n_heads, kd, vd, window, scale2, n_splits)
     if (kd <= 96 && vd <= 64) GO(3, 4);
     else if (kd <= 160 && vd <= 128) GO(5, 8);
-    else GO(9, 16);
+    else if (kd <= 288 && vd <= 256) GO(9, 16);
+    else GO(18, 32);
 #undef GO
     GI_CHECK_LAUNCH("latent_attention");
     if (n_splits > 1) {

@@ -248,8 +248,11 @@ __device__ __forceinline__ int rows_before(const int* __restrict__ slot, const i
 //   items 2 n_kv .. + n_heads a value head: convolution, SiLU
 //   the last item             per head the decay exp(-exp(a_log) softplus(pre_a + dt_bias)) and the step size sigmoid(pre_b)
 // qkv: float32 [rows, n_conv] in the columns' order; gates: float32 [rows, 2 n_heads], decays then step sizes.
+// move_tail: every row of the step is its request's only one (a decode step); the thread that has read a channel's tail then also
+// moves it on by the row's own input, and no other kernel needs to (with several rows of a request in a step, rows read the tail
+// that others would be writing: `delta_tail_kernel` does it behind this one).
 __global__ __launch_bounds__(64) void delta_prepare_kernel(const float* __restrict__ proj, long ld, int conv_off, int a_off, int b_off,
-                                                          const float* __restrict__ taps, int n_taps, const float* __restrict__ tail, long tail_stride,
+                                                          const float* __restrict__ taps, int n_taps, float* __restrict__ tail, long tail_stride, int move_tail,
                                                           const float* __restrict__ a_log, const float* __restrict__ dt_bias,
                                                           const int* __restrict__ slot, const int* __restrict__ pos, float* __restrict__ qkv,
                                                           float* __restrict__ gates, int n_heads, int n_kv, int dk, int dv, float q_scale) {
@@ -266,7 +269,7 @@ __global__ __launch_bounds__(64) void delta_prepare_kernel(const float* __restri
     const bool unit = item < 2 * n_kv;
     const int first = unit ? item * dk : 2 * n_kv * dk + (item - 2 * n_kv) * dv, width = unit ? dk : dv;
     const int before = rows_before(slot, pos, t, n_taps - 1);
-    const float* old = tail + (size_t)slot[t] * tail_stride;
+    float* old = tail + (size_t)slot[t] * tail_stride;
     float ss = 0.f;
     for (int d = lane; d < width; d += 64) {
         const int c = first + d;
@@ -275,6 +278,10 @@ __global__ __launch_bounds__(64) void delta_prepare_kernel(const float* __restri
             const int back = n_taps - 1 - j;                      // rows before t that tap j reads
             const float x = back <= before ? proj[(size_t)(t - back) * ld + conv_off + c] : old[(size_t)(n_taps - 1 - (back - before)) * n_conv + c];
             y = fmaf(taps[(size_t)c * n_taps + j], x, y);
+        }
+        if (move_tail) {
+            for (int i = 0; i + 2 < n_taps; ++i) old[(size_t)i * n_conv + c] = old[(size_t)(i + 1) * n_conv + c];
+            if (n_taps > 1) old[(size_t)(n_taps - 2) * n_conv + c] = proj[(size_t)t * ld + conv_off + c];
         }
         y = y / (1.0f + expf(-y));
         qkv[(size_t)t * n_conv + c] = y;                          // (read back below by the lane that wrote it)
@@ -458,7 +465,7 @@ GI_API int gi_delta_max_taps() { return DELTA_MAX_TAPS; }
 // proj: float32 [n_rows, ld]; see delta_prepare_kernel.  state: [slots, state_stride], a slot's memories then its tail.
 GI_API int gi_delta_prepare(const float* proj, long ld, int conv_off, int a_off, int b_off, const float* taps, int n_taps, const float* a_log,
                             const float* dt_bias, const int* slot, const int* pos, float* state, long state_stride, float* qkv, float* gates,
-                            int n_rows, int n_heads, int n_kv, int dk, int dv, float q_scale, hipStream_t stream) {
+                            int n_rows, int n_heads, int n_kv, int dk, int dv, float q_scale, int move_tail, hipStream_t stream) {
     GI_REQUIRE(n_rows > 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0 && dk > 0 && dv > 0, "delta_prepare: bad sizes (rows %d, heads %d, kv heads %d, dk %d, dv %d)",
                n_rows, n_heads, n_kv, dk, dv);
     GI_REQUIRE(n_taps >= 1 && n_taps <= DELTA_MAX_TAPS, "delta_prepare: %d taps, 1 to %d are served", n_taps, DELTA_MAX_TAPS);
@@ -467,7 +474,7 @@ GI_API int gi_delta_prepare(const float* proj, long ld, int conv_off, int a_off,
                "delta_prepare: the columns named lie outside the rows");
     GI_REQUIRE(state_stride >= gi_delta_state_floats(n_heads, n_kv, dk, dv, n_taps) && 2 * n_kv + n_heads + 1 <= 65535, "delta_prepare: state stride %ld too small, or too many heads", state_stride);
     dim3 grid(n_rows, 2 * n_kv + n_heads + 1);
-    delta_prepare_kernel<<<grid, 64, 0, stream>>>(proj, ld, conv_off, a_off, b_off, taps, n_taps, state + gi_delta_memory_floats(n_heads, dk, dv), state_stride,
+    delta_prepare_kernel<<<grid, 64, 0, stream>>>(proj, ld, conv_off, a_off, b_off, taps, n_taps, state + gi_delta_memory_floats(n_heads, dk, dv), state_stride, move_tail,
                                                   a_log, dt_bias, slot, pos, qkv, gates, n_heads, n_kv, dk, dv, q_scale);
     GI_CHECK_LAUNCH("delta_prepare");
     return 0;

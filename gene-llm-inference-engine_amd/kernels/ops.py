@@ -43,7 +43,7 @@ _SIGNATURES = {
                            c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_long, c_void_p],
     "gi_xielu": [c_void_p, c_long, c_void_p, c_int, c_long, c_int, c_int, c_void_p, c_void_p],
     "gi_delta_prepare": [c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p,
-                         c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+                         c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
     "gi_delta_tail": [c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p],
     "gi_delta_scan": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_long, c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p],
     "gi_latent_prepare": [c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
@@ -678,12 +678,14 @@ def _delta_checks(what, proj, state, n_heads, n_kv, dk, dv, n_taps):
         raise KernelError(f"{what}: keys of 1 to {DELTA_MAX_KEY_DIM} channels, 1 to {DELTA_MAX_TAPS} taps and heads in whole groups are served")
 
 
-def delta_prepare(proj, conv_off, a_off, b_off, taps, a_log, dt_bias, ctx_slots, ctx_positions, state, qkv, gates, n_heads, n_kv, dk, dv, q_scale):
+def delta_prepare(proj, conv_off, a_off, b_off, taps, a_log, dt_bias, ctx_slots, ctx_positions, state, qkv, gates, n_heads, n_kv, dk, dv, q_scale,
+                  single_rows=False):
     """What the gated delta rule needs of every row (csrc/recurrent.hip: delta_prepare_kernel): the columns [conv_off, conv_off +
     2 n_kv dk + n_heads dv) of proj (queries, keys, values) through their short convolutions (taps float32 [channels, n_taps]; a
     request's rows before this step come from its state) and SiLU, queries and keys made unit vectors per head (queries times
     q_scale), into qkv float32 [n, channels]; and gates float32 [n, 2 heads]: the decays exp(-exp(a_log) softplus(proj[a_off + h] +
-    dt_bias)), then the step sizes sigmoid(proj[b_off + h])."""
+    dt_bias)), then the step sizes sigmoid(proj[b_off + h]).  single_rows: every row is its request's only row of the step; the
+    kernel then also moves every request's tail on by its row, and `delta_tail` is not needed."""
     _dev(proj, taps, a_log, dt_bias, ctx_slots, ctx_positions, state, qkv, gates)
     n, n_conv = proj.shape[0], 2 * n_kv * dk + n_heads * dv
     n_taps = taps.shape[1]
@@ -701,7 +703,7 @@ def delta_prepare(proj, conv_off, a_off, b_off, taps, a_log, dt_bias, ctx_slots,
     _i32(ctx_positions, "delta_prepare: positions", n)
     _call("gi_delta_prepare", proj.data_ptr(), proj.stride(0), int(conv_off), int(a_off), int(b_off), taps.data_ptr(), n_taps, a_log.data_ptr(), dt_bias.data_ptr(),
           ctx_slots.data_ptr(), ctx_positions.data_ptr(), state.data_ptr(), state.stride(0), qkv.data_ptr(), gates.data_ptr(), n, n_heads, n_kv, dk, dv,
-          float(q_scale), _stream())
+          float(q_scale), 1 if single_rows else 0, _stream())
 
 
 def delta_tail(proj, conv_off, n_taps, seg_start, seg_len, row_slot, state, n_heads, n_kv, dk, dv):

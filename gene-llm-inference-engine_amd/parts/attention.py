@@ -17,7 +17,7 @@ from ..cache.needs import PagedKvNeed
 from ..kernels import ops
 from ..weights.loader import TensorNeed
 from .base import Mixer, PositionEncoding, position_class, register_mixer
-from .linear import activation_dtype_for, linear, linear_onto
+from .linear import activation_dtype_for, linear, linear_onto, takes_handed_norm
 from .norm import HandedRows, NormedRows
 from .rope import rotation_tables
 
@@ -167,7 +167,9 @@ class Attention(Mixer):
         return PagedKvNeed(spec.n_kv_heads, spec.head_dim, spec.window, None if spec.value_dim in (None, spec.head_dim) else spec.value_dim, spec.keep_chunk)
 
     def takes_handed_norm(self, n_rows: int) -> bool:
-        if self.in_dtype != torch.bfloat16 or self.general:
+        if self.in_dtype == torch.bfloat16 and self.general:          # (the general path's one product goes through `linear`)
+            return takes_handed_norm(self.w_qkv, n_rows)
+        if self.in_dtype != torch.bfloat16:
             return False
         if ops.gemm_bf16_takes_norm(n_rows, self.w_qkv.shape[0], self.w_qkv.shape[1]):
             return True

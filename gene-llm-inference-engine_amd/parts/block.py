@@ -169,9 +169,26 @@ class SandwichBlock:
 register_block("sandwich", SandwichBlock)
 
 
+class _Readers:
+    """The parts that read one norm's rows, asked as one whether they take that norm half applied."""
+
+    def __init__(self, parts):
+        self.parts = parts
+        self.accepts_deferred_norm = all(getattr(p, "accepts_deferred_norm", False) for p in parts)
+        dtypes = {getattr(p, "in_dtype", None) for p in parts}
+        self.in_dtype = dtypes.pop() if len(dtypes) == 1 else None
+
+    def takes_handed_norm(self, n_rows: int) -> bool:
+        return self.in_dtype is not None and all(hasattr(p, "takes_handed_norm") and p.takes_handed_norm(n_rows) for p in self.parts)
+
+
 class ParallelBlock:
     """x += mixer(h) + feed_forward(h) with h = norm_1(x): both halves read the same normed rows, which are made once, and each
-    adds its result onto x (the two sums reach x one after the other; neither half reads x)."""
+    adds its result onto x (the two sums reach x one after the other; neither half reads x).  The block plays the game of
+    handing a norm on (`hands_norm_on`, `first_reader`, `handed`, `next_reader`): the half that writes x last does the next
+    norm's first share, and a norm so handed to this block is finished by the first products of both halves, where both can
+    (asked beforehand: the second half must not fall back on rows that the first has changed by then)."""
+    hands_norm_on = True
 
     def __init__(self, spec, tensors, dtype, device):
         self.spec = spec
@@ -180,6 +197,7 @@ class ParallelBlock:
         self.mixer_norm = norm_class(spec.mixer_norm)(spec.mixer_norm, tensors, dtype, device)
         self.mixer = mixer_class(spec.mixer)(spec.mixer, tensors, dtype, device)
         self.feed_forward = None if spec.feed_forward is None else feed_forward_class(spec.feed_forward)(spec.feed_forward, tensors, dtype, device)
+        self._readers = _Readers(self._parts()[1:])
 
     def _parts(self):
         return [self.mixer_norm, self.mixer] + ([self.feed_forward] if self.feed_forward is not None else [])
@@ -199,21 +217,30 @@ class ParallelBlock:
     def cache_need(cls, spec):
         return mixer_class(spec.mixer).cache_need(spec.mixer)
 
-    def forward(self, x, ctx, cache):
-        dtypes = {getattr(p, "in_dtype", ctx.dtype) for p in self._parts()[1:]}
-        if len(dtypes) == 1:                      # one set of normed rows serves both halves
-            h = self.mixer_norm(x, dtypes.pop())
+    def first_reader(self):
+        return self.mixer_norm, self._readers
+
+    def forward(self, x, ctx, cache, handed=None, next_reader=None):
+        """handed: this block's norm as whoever wrote x last left it (half applied), or None.  next_reader: `first_reader()` of
+        whatever reads x after this block, or None.  Returns that reader's norm handed on, or None."""
+        if handed is not None and handed.norm is self.mixer_norm and self._readers.takes_handed_norm(ctx.n_rows):
+            rows = lambda part: handed
+        elif self._readers.in_dtype is not None:      # one set of normed rows serves both halves
+            h = self.mixer_norm(x, self._readers.in_dtype)
             rows = lambda part: h
         else:
-            rows = lambda part: self.mixer_norm(x, getattr(part, "in_dtype", ctx.dtype))
-        h_ff = rows(self.feed_forward) if self.feed_forward is not None else None      # (made before the mixer changes x)
-        self.mixer.forward(rows(self.mixer), x, ctx, cache)
+            made = {part: self.mixer_norm(x, getattr(part, "in_dtype", ctx.dtype)) for part in self._parts()[1:]}      # (before anything changes x)
+            rows = made.__getitem__
+        last = self.feed_forward if self.feed_forward is not None else self.mixer
+        then = norm_to_hand_on(next_reader, ctx.n_rows) if getattr(last, "hands_norm_on", False) else None
+        out = self.mixer.forward(rows(self.mixer), x, ctx, cache, then=then) if last is self.mixer and then is not None else self.mixer.forward(rows(self.mixer), x, ctx, cache)
         if ctx.trace is not None:
             ctx.trace("attn_out", x)
         if self.feed_forward is not None:
-            self.feed_forward.forward(h_ff, x, ctx)
+            out = self.feed_forward.forward(rows(self.feed_forward), x, ctx, then=then) if then is not None else self.feed_forward.forward(rows(self.feed_forward), x, ctx)
         if ctx.trace is not None:
             ctx.trace("ffn_out", x)
+        return out if then is not None else None
 
 
 register_block("parallel", ParallelBlock)

@@ -3,7 +3,7 @@
 One product with the stacked matrix [q; k; v; output gate; a; b] gives the 32-bit projections of a step's rows.  One kernel
 makes of them what the rule reads: q, k and v through their short convolutions (a request's rows before this step come from
 its state) and SiLU, q and k as unit vectors, the decays and step sizes.  One kernel keeps every request's last rows for the
-next step's convolutions.  One kernel steps the memories over every request's rows, in order, from the request's state slot
+next step's convolutions (in a step of single rows the kernel before it does that on its way).  One kernel steps the memories over every request's rows, in order, from the request's state slot
 and back into it.  One kernel divides every head's read-out by its root mean square, multiplies by the norm's weights and by
 SiLU of the output gate, and stores the rows as the output product reads them.  Everything between the projections and the
 output product is 32-bit, whatever the compute dtype.
@@ -20,13 +20,17 @@ from ..kernels import ops
 from ..weights.loader import TensorNeed
 from .attention import _pad_rows
 from .base import Mixer, register_mixer
-from .linear import activation_dtype_for, linear, linear_onto
+from .linear import activation_dtype_for, linear, linear_onto, takes_handed_norm
 
 
 class GatedDelta(Mixer):
     graph_safe = True
     accepts_deferred_norm = True      # its input goes into `linear` only
+    hands_norm_on = True              # `forward` takes `then`, the norm that reads the residual next
     can_overwrite = True
+
+    def takes_handed_norm(self, n_rows: int) -> bool:
+        return self.in_dtype == torch.bfloat16 and takes_handed_norm(self.w_in, n_rows)
 
     def __init__(self, spec, tensors, dtype, device):
         super().__init__(spec, tensors, dtype, device)
@@ -65,7 +69,7 @@ class GatedDelta(Mixer):
     def cache_need(cls, spec):
         return StateNeed((ops.delta_state_floats(spec.n_heads, spec.n_kv_heads, spec.key_dim, spec.value_dim, spec.conv_taps),), torch.float32)
 
-    def forward(self, h, residual, ctx, cache, overwrite=False):
+    def forward(self, h, residual, ctx, cache, then=None, overwrite=False):
         s, T, o, dev = self.spec, ctx.n_rows, self.offsets, ctx.device
         H, G, dk, dv = s.n_heads, s.n_kv_heads, s.key_dim, s.value_dim
         vv = H * dv
@@ -74,17 +78,19 @@ class GatedDelta(Mixer):
         seg_start, seg_len = ops.segments(ctx)
         qkv = torch.empty((T, 2 * G * dk + vv), dtype=torch.float32, device=dev)
         gates = torch.empty((T, 2 * H), dtype=torch.float32, device=dev)
+        single_rows = ctx.max_seg_len == 1            # (a step's shape, which a captured pass shares with its replays)
         ops.delta_prepare(proj, o["conv"], o["a"], o["b"], self.taps, self.a_log, self.dt_bias, ctx.row_slot, ctx.row_pos, cache.state, qkv, gates,
-                          H, G, dk, dv, dk ** -0.5)
-        ops.delta_tail(proj, o["conv"], s.conv_taps, seg_start, seg_len, ctx.row_slot, cache.state, H, G, dk, dv)
+                          H, G, dk, dv, dk ** -0.5, single_rows)
+        if not single_rows:
+            ops.delta_tail(proj, o["conv"], s.conv_taps, seg_start, seg_len, ctx.row_slot, cache.state, H, G, dk, dv)
         read = torch.empty((T, vv), dtype=torch.float32, device=dev)
         ops.delta_scan(qkv, gates, seg_start, seg_len, ctx.row_slot, cache.state, read, H, G, dk, dv)
         mid = torch.empty((T, vv), dtype=self.mid_dtype, device=dev)
         ops.head_norm_gate(read, proj[:, o["g"]:o["g"] + vv], self.out_norm, s.norm_eps, mid, H, dv, gate_activation="silu")
         if overwrite:
             linear(mid, self.w_o, residual)
-        else:
-            linear_onto(mid, self.w_o, residual)
+            return None
+        return linear_onto(mid, self.w_o, residual, then)
 
 
 register_mixer("gated_delta", GatedDelta)

@@ -23,7 +23,7 @@ from ..kernels import ops
 from ..weights.loader import TensorNeed
 from .attention import _pad_rows
 from .base import Mixer, position_class, register_mixer
-from .linear import activation_dtype_for, linear, linear_onto
+from .linear import activation_dtype_for, linear, linear_onto, takes_handed_norm
 
 
 def _head_product(a, w, out):
@@ -47,7 +47,11 @@ def heads_product(a, w, out, n_heads, out_head_stride=None):
 
 class LatentAttention(Mixer):
     accepts_deferred_norm = True      # its input goes into `linear` only
+    hands_norm_on = True              # `forward` takes `then`, the norm that reads the residual next
     can_overwrite = True
+
+    def takes_handed_norm(self, n_rows: int) -> bool:
+        return self.in_dtype == torch.bfloat16 and takes_handed_norm(self.w_down, n_rows)
 
     def __init__(self, spec, tensors, dtype, device):
         super().__init__(spec, tensors, dtype, device)
@@ -92,7 +96,7 @@ class LatentAttention(Mixer):
     def cache_need(cls, spec):
         return PagedKvNeed(1, spec.kv_rank + spec.rotary_dim, spec.window, spec.kv_rank, None)
 
-    def forward(self, h, residual, ctx, cache, overwrite=False):
+    def forward(self, h, residual, ctx, cache, then=None, overwrite=False):
         s, T, dev = self.spec, ctx.n_rows, ctx.device
         H, kd = s.n_heads, self.key_dim
         down = torch.empty((T, self.w_down.shape[0]), dtype=torch.float32, device=dev)
@@ -119,8 +123,8 @@ class LatentAttention(Mixer):
         heads_product(attended, self.w_uv, att, H)
         if overwrite:
             linear(att, self.w_o, residual)
-        else:
-            linear_onto(att, self.w_o, residual)
+            return None
+        return linear_onto(att, self.w_o, residual, then)
 
 
 register_mixer("latent_attention", LatentAttention)

@@ -49,6 +49,15 @@ def linear_onto(a: torch.Tensor, weight: torch.Tensor, residual: torch.Tensor, t
     return None
 
 
+def takes_handed_norm(weight: torch.Tensor, n_rows: int, gated: bool = False) -> bool:
+    """Whether `linear(handed rows, weight, ...)` finishes a norm handed on at this number of rows, rather than asking for the rows
+    normed the ordinary way: exactly `linear`'s own conditions, for parts that must know beforehand (a part that reads normed
+    rows after another part has changed the rows they were made of cannot fall back on them)."""
+    n, k = weight.shape
+    return (weight.dtype == torch.bfloat16 and k % 8 == 0 and weight.stride(1) == 1 and weight.stride(0) % 8 == 0 and weight.data_ptr() % 16 == 0
+            and ops.gemm_bf16_takes_norm(n_rows, n, k, gated))
+
+
 def activation_dtype_for(weight: torch.Tensor, compute_dtype: torch.dtype) -> torch.dtype:
     """What the input of a product with `weight` is stored as: bfloat16 only if both the compute
     dtype and the weight are; a weight kept in 32-bit gets 32-bit activations."""

@@ -8,7 +8,7 @@ import torch
 from ..kernels import ops
 from ..weights.loader import TensorNeed
 from .base import FeedForward, register_feed_forward
-from .linear import activation_dtype_for, linear, linear_onto
+from .linear import activation_dtype_for, linear, linear_onto, takes_handed_norm
 
 
 class SwiGlu(FeedForward):
@@ -63,7 +63,11 @@ class DenseMlp(FeedForward):
     product's rows, which it stores as the down product reads them."""
     graph_safe = True
     accepts_deferred_norm = True      # its input goes into `linear` only
+    hands_norm_on = True              # `forward` takes `then`, the norm that reads the residual next
     can_overwrite = True
+
+    def takes_handed_norm(self, n_rows: int) -> bool:
+        return self.in_dtype == torch.bfloat16 and takes_handed_norm(self.w_up, n_rows)
 
     def __init__(self, spec, tensors, dtype, device):
         super().__init__(spec, tensors, dtype, device)
@@ -81,14 +85,16 @@ class DenseMlp(FeedForward):
         i, d = spec.intermediate_size, spec.hidden_size
         return [TensorNeed(spec.up_proj, (i, d)), TensorNeed(spec.down_proj, (d, i)), TensorNeed(spec.activation_params, (2,))]
 
-    def forward(self, h, residual, ctx, overwrite=False):
+    def forward(self, h, residual, ctx, then=None, overwrite=False):
         T, inter = ctx.n_rows, self.spec.intermediate_size
         up = torch.empty((T, inter), dtype=torch.float32, device=ctx.device)
         linear(h, self.w_up, up)
         mid = torch.empty((T, inter), dtype=self.mid_dtype, device=ctx.device)
         ops.xielu(up, mid, self.params)
-        linear(mid, self.w_down, residual, accumulate=not overwrite)
-        return None
+        if overwrite:
+            linear(mid, self.w_down, residual)
+            return None
+        return linear_onto(mid, self.w_down, residual, then)
 
 
 register_feed_forward("dense_mlp", DenseMlp)
