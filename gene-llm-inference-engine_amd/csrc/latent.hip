@@ -240,24 +240,33 @@ __global__ __launch_bounds__(64) void latent_attention_kernel(const bf16_t* __re
         }
 }
 
-// The shares of one (row, head), in their order: out = sum_s 2^(m_s - m) o_s / sum_s 2^(m_s - m) l_s.
+// The shares of one (row, head): out = sum_s 2^(m_s - m) o_s / sum_s 2^(m_s - m) l_s.  Lane s fetches share s's maximum and sum (all
+// at once, not one behind the other); the weights wait in LDS; a lane then adds its channels over the shares, in their order, eight
+// loads in flight.
 __global__ __launch_bounds__(64) void latent_merge_kernel(const float* __restrict__ part, bf16_t* __restrict__ out, int vd, int n_splits) {
+    __shared__ float weight[64];
     const size_t rh = blockIdx.x;
+    const int lane = threadIdx.x;
     const float* mine = part + rh * n_splits * (vd + 2);
-    float m = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) m = fmaxf(m, mine[(size_t)s * (vd + 2)]);
-    float l = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-        const float ms = mine[(size_t)s * (vd + 2)];
-        if (ms != -INFINITY) l += exp2_fast(ms - m) * mine[(size_t)s * (vd + 2) + 1];
-    }
-    for (int c = threadIdx.x; c < vd; c += 64) {
+    const float ms = lane < n_splits ? mine[(size_t)lane * (vd + 2)] : -INFINITY;
+    const float ls = lane < n_splits ? mine[(size_t)lane * (vd + 2) + 1] : 0.f;
+    const float m = wave_max(ms);
+    const float w = ms == -INFINITY ? 0.f : exp2_fast(ms - m);
+    const float inv = 1.0f / wave_sum(w * ls);
+    weight[lane] = w;
+    __syncthreads();
+    for (int c = lane; c < vd; c += 64) {
         float acc = 0.f;
-        for (int s = 0; s < n_splits; ++s) {
-            const float ms = mine[(size_t)s * (vd + 2)];
-            if (ms != -INFINITY) acc = fmaf(exp2_fast(ms - m), mine[(size_t)s * (vd + 2) + 2 + c], acc);
+        int s = 0;
+        for (; s + 8 <= n_splits; s += 8) {
+            float v[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = mine[(size_t)(s + e) * (vd + 2) + 2 + c];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc = fmaf(weight[s + e], v[e], acc);
         }
-        out[rh * vd + c] = f32_to_bf16(acc / l);
+        for (; s < n_splits; ++s) acc = fmaf(weight[s], mine[(size_t)s * (vd + 2) + 2 + c], acc);
+        out[rh * vd + c] = f32_to_bf16(acc * inv);
     }
 }
 

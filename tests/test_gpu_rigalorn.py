@@ -512,6 +512,18 @@ def test_replay_through_the_command_line(folders, tmp_path, dtype, mode):
             assert_within_bfloat16_noise(mine, lambda p: exact[p], lambda p: rounded[p], f"replay {mode} {rid}")
 
 
+def test_generation_from_the_command_line_on_random_weights():
+    """bin/gi_generate on the shipped example configuration, random weights, greedy: runs, and twice the same."""
+    import subprocess
+    from pathlib import Path
+    root = Path(__file__).resolve().parent.parent
+    cmd = [str(root / "bin" / "gi_generate"), "--config", str(root / "configs" / "rigalorn-small.json"), "--random-seed", "3", "--prompt-ids", "5 17 3 999 4",
+           "--steps", "24", "--temperature", "0"]
+    runs = [subprocess.run(cmd, capture_output=True, text=True, timeout=280) for _ in range(2)]
+    assert all(r.returncode == 0 for r in runs), runs[0].stderr[-2000:]
+    assert runs[0].stdout == runs[1].stdout and len(runs[0].stdout.split()) >= 20
+
+
 def test_the_new_parts_serve_other_designs():
     """The parts are not Rigalorn's own: a model put together by hand, a pre-norm layer around the gated delta rule and a SiLU-gated
     feed-forward, and a parallel layer around a plain Llama attention and the feed-forward without a gate, through the same step
