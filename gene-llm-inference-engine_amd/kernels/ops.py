@@ -49,8 +49,9 @@ _SIGNATURES = {
     "gi_latent_prepare": [c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                           c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_int, c_int, c_void_p],
     "gi_heads_product": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_long, c_long, c_int, c_int, c_int, c_int, c_void_p],
-    "gi_latent_attention_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int,
+    "gi_latent_attention_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int,
                                  c_float, c_int, c_void_p],
+    "gi_latent_attention_tiles_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "gi_latent_queries": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gi_act_mul": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "gi_segments": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p],
@@ -114,6 +115,10 @@ def lib():
         l.gi_mlstm_max_key_dim.restype = c_int
         l.gi_latent_attention_supports.argtypes = [c_int, c_int, c_int]
         l.gi_latent_attention_supports.restype = c_int
+        l.gi_latent_attention_tiles_supports.argtypes = [c_int, c_int, c_int, c_int]
+        l.gi_latent_attention_tiles_supports.restype = c_int
+        l.gi_latent_attention_tiles_prepare.argtypes = []
+        l.gi_latent_attention_tiles_prepare.restype = c_int
         l.gi_probe_mfma_flops.argtypes = [c_int, c_int]
         l.gi_probe_mfma_flops.restype = c_long
         _lib = l
@@ -1343,10 +1348,18 @@ def latent_attention_bf16_supports(kd, vd, page_size) -> bool:
     return bool(lib().gi_latent_attention_supports(kd, vd, page_size))
 
 
+def latent_attention_prepare():
+    """Once, outside any captured pass: the prompt kernel's LDS (more than the default limit) is asked for."""
+    if lib().gi_latent_attention_tiles_prepare() != 0:
+        raise KernelError(lib().gi_last_error().decode())
+
+
 def latent_attention_bf16(q, cache, out, ctx, table, n_heads, kd, vd, page_size, window=None, scale=1.0):
     """Attention of a step's rows over latent pages (one key/value head for all query heads: keys [place][kd], then the values
-    [vd][place]) on the matrix cores; q bfloat16 [n, heads*kd], out bfloat16 [n, heads*vd].  Every row is a wave per 16 heads and
-    share of its context; with few rows the context is shared out further and a second kernel adds the shares."""
+    [vd][place]) on the matrix cores; q bfloat16 [n, heads*kd], out bfloat16 [n, heads*vd].  The rows of prompts go by the attention
+    plan's tiles: a workgroup takes a few consecutive rows with all their heads and stages the keys they see once in LDS.  Single
+    rows, and the rows of short portions, are a wave per 16 heads and share of their context each; with few of them the context is
+    shared out further and a second kernel adds the shares."""
     _dev(q, cache, out, table)
     n = q.shape[0]
     if not (q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and q.shape == (n, n_heads * kd) and q.is_contiguous()
@@ -1355,14 +1368,22 @@ def latent_attention_bf16(q, cache, out, ctx, table, n_heads, kd, vd, page_size,
     _check_paged(cache, table, "latent_attention")
     _i32(ctx.row_pos, "latent_attention: positions", n)
     _i32(ctx.row_slot, "latent_attention: slots", n)
-    plan = _plan_of(ctx)                  # (its longest context is the bracket's in a captured pass: the same for every replay)
-    span = max(plan.max_decode_context, plan.max_tile_context, 1)
+    plan = _plan_of(ctx)                  # (its longest contexts are the bracket's in a captured pass: the same for every replay)
+    by_tiles = plan.n_tiles > 0 and bool(lib().gi_latent_attention_tiles_supports(n_heads, kd, vd, int(page_size)))
+    if by_tiles:
+        _call("gi_latent_attention_tiles_bf16", q.data_ptr(), cache.data_ptr(), out.data_ptr(), plan.tiles.data_ptr(), plan.n_tiles, plan.tile, table.data_ptr(),
+              table.stride(0), cache.stride(0), int(page_size), n_heads, kd, vd, int(window or 0), float(scale), _stream())
+        if not plan.n_decode:
+            return out
+        n_single, rows, span = plan.n_decode, plan.decode_rows, plan.max_decode_context
+    else:
+        n_single, rows, span = n, None, max(plan.max_decode_context, plan.max_tile_context, 1)
     if window:
         span = min(span, int(window) + 31)
-    groups = n * (-(-n_heads // 16))
+    groups = n_single * (-(-n_heads // 16))
     n_splits = max(1, min(16, 2048 // groups, (span + 63) // 64))
-    n_part = n * n_heads * n_splits * (vd + 2) if n_splits > 1 else 0
+    n_part = n_single * n_heads * n_splits * (vd + 2) if n_splits > 1 else 0
     part = torch.empty(n_part, dtype=torch.float32, device=out.device) if n_part else None
-    _call("gi_latent_attention_bf16", q.data_ptr(), cache.data_ptr(), out.data_ptr(), _ptr(part), n_part, ctx.row_pos.data_ptr(), ctx.row_slot.data_ptr(), table.data_ptr(),
-          table.stride(0), cache.stride(0), int(page_size), n, n_heads, kd, vd, int(window or 0), float(scale), n_splits, _stream())
+    _call("gi_latent_attention_bf16", q.data_ptr(), cache.data_ptr(), out.data_ptr(), _ptr(part), n_part, _ptr(rows), ctx.row_pos.data_ptr(), ctx.row_slot.data_ptr(),
+          table.data_ptr(), table.stride(0), cache.stride(0), int(page_size), n_single, n_heads, kd, vd, int(window or 0), float(scale), n_splits, _stream())
     return out

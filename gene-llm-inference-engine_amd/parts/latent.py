@@ -80,6 +80,8 @@ class LatentAttention(Mixer):
         self.plain_dtype = activation_dtype_for(self.w_uk_t, dtype)
         self.att_dtype = activation_dtype_for(self.w_o, dtype)
         self.graph_safe = self.position is None or bool(getattr(self.position, "graph_safe", False))
+        if dtype == torch.bfloat16 and torch.device(device).type == "cuda":
+            ops.latent_attention_prepare()
 
     def weights_read_per_step(self):
         return [self.w_down, self.q_norm, self.kv_norm, self.w_uq, self.w_uk_t, self.w_uv, self.w_o]

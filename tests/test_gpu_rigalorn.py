@@ -258,7 +258,8 @@ def test_attention_through_latents_against_keys_and_values_made_in_full(T, windo
 
 @pytest.mark.parametrize("H, kd, vd, window, lens, pos0", [(20, 144, 128, 40, [1, 1, 1], [700, 39, 0]), (8, 80, 64, None, [130, 1], [0, 300]), (32, 288, 256, 100, [70], [50]),
                                                           (3, 24, 16, 17, [33, 2, 1], [15, 16, 17]), (16, 96, 64, 1, [20], [0]), (16, 576, 512, 48, [40, 1], [30, 200]),
-                                                          (5, 296, 264, None, [3], [60])])
+                                                          (5, 296, 264, None, [3], [60]), (16, 576, 512, 48, [100, 1], [30, 200]), (20, 144, 128, 40, [130, 70, 1], [700, 0, 5]),
+                                                          (40, 80, 64, None, [90], [10]), (8, 288, 256, 300, [129, 200], [77, 0]), (130, 32, 16, 20, [80], [3])])
 def test_matrix_core_attention_over_latent_pages(H, kd, vd, window, lens, pos0):
     """Requests at other positions each, on shuffled pages: single rows whose context is shared out over several waves, and
     portions of prompts; heads that fill one and a half matrix instructions; keys that are no multiple of 32 channels.  One key
