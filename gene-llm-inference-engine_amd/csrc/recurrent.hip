@@ -230,7 +230,7 @@ __global__ __launch_bounds__(64) void head_norm_gate_kernel(const float* __restr
 
 
 // ------------------------------------------------------------------------------------- gated delta rule
-constexpr int DELTA_MAX_TAPS = 8;
+constexpr int DELTA_MAX_TAPS = 16;
 
 __device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 

@@ -659,7 +659,7 @@ def head_norm_gate(o, gate, weight, eps, out, n_heads, dv, den=None, gate_activa
 
 
 # ------------------------------------------------------------------------------------------------ the gated delta rule
-DELTA_MAX_KEY_DIM, DELTA_MAX_TAPS = 512, 8
+DELTA_MAX_KEY_DIM, DELTA_MAX_TAPS = 512, 16
 
 
 def delta_memory_floats(n_heads, dk, dv) -> int:

@@ -96,7 +96,7 @@ def test_activation_of_the_plain_feed_forward():
         assert torch.equal(half.cpu(), out.cpu().to(torch.bfloat16))
 
 
-@pytest.mark.parametrize("heads, kv, dk, dv, taps", [(4, 2, 16, 24, 4), (3, 3, 64, 64, 2), (2, 1, 130, 10, 5), (1, 1, 7, 201, 1), (5, 5, 3, 5, 3), (2, 2, 300, 6, 8)])
+@pytest.mark.parametrize("heads, kv, dk, dv, taps", [(4, 2, 16, 24, 4), (3, 3, 64, 64, 2), (2, 1, 130, 10, 5), (1, 1, 7, 201, 1), (5, 5, 3, 5, 3), (2, 2, 300, 6, 8), (1, 1, 20, 9, 13)])
 def test_gated_delta_rule_kernels(heads, kv, dk, dv, taps):
     """Two requests of unequal length in one step; then the longer one again from a fresh slot in steps down to one and two rows:
     the memories and the convolutions' tails carry, and the bits do not change."""
@@ -405,6 +405,39 @@ def test_mixed_batches_on_a_pool_that_is_used_again(folders, name, dtype):
         else:
             exact, rounded = plain_logits(folders, name, tokens), plain_logits(folders, name, tokens, rounded=True)
             assert_within_bfloat16_noise(mine, lambda p: exact[p], lambda p: rounded[p], f"{name} mixed {rid}")
+
+
+@pytest.mark.parametrize("name, dtype", [("C", "bfloat16"), ("C", "float32"), ("B", "float32")])
+def test_long_portions_beside_single_rows(folders, name, dtype):
+    """Steps that hold portions of a hundred rows and more of some requests (the kernels that take the rows of prompts tile by tile)
+    beside single rows and short portions of others, every request at another position."""
+    from geneinfer_amd.engine import StepEntry
+    cfg = CONFIGS[name]
+    tokens = {r: _prompt(cfg, n, 70 + n) for r, n in (("a", 330), ("b", 150), ("c", 171), ("d", 40))}
+    schedule = [[("a", 100), ("c", 70)], [("a", 130), ("b", 1), ("c", 1)], [("b", 140), ("a", 1), ("c", 99), ("d", 3)], [("a", 99), ("b", 2), ("c", 1), ("d", 37)], [("b", 7)]]
+    runner = make_runner(folders, name, dtype, max_tokens=1024, max_requests=4)
+    at, got = {r: 0 for r in tokens}, {r: [] for r in tokens}
+    for step in schedule:
+        entries = []
+        for r, n in step:
+            if not runner.is_open(r):
+                runner.open(r)
+            entries.append(StepEntry(r, tokens[r][at[r]:at[r] + n], tuple(range(n))))
+        logits = runner.step(entries).cpu()
+        row = 0
+        for r, n in step:
+            got[r].append(logits[row:row + n])
+            row += n
+            at[r] += n
+    assert all(at[r] == len(t) for r, t in tokens.items())
+    alone = make_runner(folders, name, dtype)
+    for r, t in tokens.items():
+        mine = torch.cat(got[r])
+        if dtype == "float32":
+            alone.open(r)
+            assert torch.equal(mine, feed(alone, r, t, [len(t)])), f"{name} {r}: a mixed step changed the logits"
+            alone.close(r)
+        check_against_plain(folders, name, dtype, t, mine, f"{name} {r} in mixed steps")
 
 
 def test_long_decoding_carries_state_and_passes_windows(folders):
