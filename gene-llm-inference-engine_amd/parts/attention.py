@@ -177,11 +177,13 @@ class Attention(Mixer):
         half_split = self.position is None or getattr(type(self.position), "half_split_tables", None) is not PositionEncoding.half_split_tables
         return half_split and ops.gemm_bf16_qkv_rope_store_takes(n_rows, self.w_qkv.shape[0], self.w_qkv.shape[1], self.spec.head_dim)
 
-    def _attend_general(self, h, ctx, cache):
+    def _attend_general(self, h, ctx, cache, projected=None):
         """The heads' outputs [rows, heads * value_dim] by the general path."""
         s, T, vd = self.spec, ctx.n_rows, self.value_dim
-        proj = torch.empty((T, self.w_qkv.shape[0]), dtype=torch.float32, device=ctx.device)
-        linear(h, self.w_qkv, proj)
+        proj = projected
+        if proj is None:
+            proj = torch.empty((T, self.w_qkv.shape[0]), dtype=torch.float32, device=ctx.device)
+            linear(h, self.w_qkv, proj)
         q, k, v = proj[:, :self.a_dim], None, None
         if s.k_proj is not None and cache.writes:
             k, v = proj[:, self.a_dim:self.a_dim + self.kv_dim], proj[:, self.a_dim + self.kv_dim:self.a_dim + self.kv_dim + s.n_kv_heads * vd]
@@ -208,10 +210,18 @@ class Attention(Mixer):
         return ops.attention_general(q_ready, cache.kv, att, ctx, cache.table, s.n_heads, s.n_kv_heads, s.head_dim, page_size=cache.page_size,
                                      value_dim=vd, window=s.window, chunk=s.chunk, scale=s.scale, sinks=self.sinks, gate=gate)
 
-    def forward(self, h, residual, ctx, cache, then=None, overwrite=False):
+    def input_weight(self):
+        """The first product's matrix, for a block that makes several parts' first products in one; None where the plain path's
+        kernels make that product themselves."""
+        return self.w_qkv if self.general and self.spec.k_proj is not None else None
+
+    def use_input_weight(self, view):
+        self.w_qkv = view
+
+    def forward(self, h, residual, ctx, cache, then=None, overwrite=False, projected=None):
         s = self.spec
         if self.general:
-            att = self._attend_general(h, ctx, cache)
+            att = self._attend_general(h, ctx, cache, projected if cache.writes else None)
             if att.dtype != self.att_dtype:
                 att = att.to(self.att_dtype)
             if overwrite:

@@ -13,6 +13,7 @@ import torch
 
 from ..kernels import ops
 from .base import feed_forward_class, mixer_class, norm_class, register_block
+from .linear import linear, takes_handed_norm
 from .norm import NormedRows, norm_to_hand_on
 
 
@@ -172,13 +173,16 @@ register_block("sandwich", SandwichBlock)
 class _Readers:
     """The parts that read one norm's rows, asked as one whether they take that norm half applied."""
 
-    def __init__(self, parts):
-        self.parts = parts
+    def __init__(self, parts, first_weight=None):
+        self.parts, self.first_weight = parts, first_weight          # first_weight(n_rows): the one matrix all of them read at this number of rows, or None
         self.accepts_deferred_norm = all(getattr(p, "accepts_deferred_norm", False) for p in parts)
         dtypes = {getattr(p, "in_dtype", None) for p in parts}
         self.in_dtype = dtypes.pop() if len(dtypes) == 1 else None
 
     def takes_handed_norm(self, n_rows: int) -> bool:
+        common = self.first_weight(n_rows) if self.first_weight is not None else None
+        if common is not None:                    # (one product for all of them)
+            return self.in_dtype == torch.bfloat16 and takes_handed_norm(common, n_rows)
         return self.in_dtype is not None and all(hasattr(p, "takes_handed_norm") and p.takes_handed_norm(n_rows) for p in self.parts)
 
 
@@ -189,6 +193,17 @@ class ParallelBlock:
     norm's first share, and a norm so handed to this block is finished by the first products of both halves, where both can
     (asked beforehand: the second half must not fall back on rows that the first has changed by then)."""
     hands_norm_on = True
+    STACK = True                     # the two halves' first products as one (off: each half makes its own)
+    # ... in steps of up to so many rows and with both matrices together up to so many bytes: one launch less a layer where launches
+    # are what a step costs (8 decoded rows, 8 layers: 0.563 -> 0.536 ms a step with 44 MB a layer); with 160 MB a layer the one product
+    # took longer than the two (1.142 -> 1.169 ms), and so did it for the rows of prompts at both sizes (5.19 -> 5.28, 11.28 -> 11.37 ms).
+    STACK_MAX_ROWS, STACK_MAX_BYTES = 128, 64 << 20
+
+    def _stacked(self, n_rows: int):
+        """The common matrix of both halves' first products, if a step of this many rows makes them as one; else None."""
+        if self.w_first is None or n_rows > self.STACK_MAX_ROWS or self.w_first.numel() * self.w_first.element_size() > self.STACK_MAX_BYTES:
+            return None
+        return self.w_first
 
     def __init__(self, spec, tensors, dtype, device):
         self.spec = spec
@@ -197,7 +212,19 @@ class ParallelBlock:
         self.mixer_norm = norm_class(spec.mixer_norm)(spec.mixer_norm, tensors, dtype, device)
         self.mixer = mixer_class(spec.mixer)(spec.mixer, tensors, dtype, device)
         self.feed_forward = None if spec.feed_forward is None else feed_forward_class(spec.feed_forward)(spec.feed_forward, tensors, dtype, device)
-        self._readers = _Readers(self._parts()[1:])
+        # Both halves begin with a product of the same rows: where both say which matrix that is (`input_weight`), the two are laid
+        # one behind the other, the block makes one product of them and hands each half its columns (`projected=`); the halves keep
+        # views of the common matrix, so nothing lies in memory twice.
+        self.w_first, self._split = None, 0
+        first = [getattr(p, "input_weight", lambda: None)() for p in (self.mixer, self.feed_forward)] if self.feed_forward is not None else []
+        if (self.STACK and len(first) == 2 and all(w is not None for w in first) and first[0].dtype == first[1].dtype and first[0].shape[1] == first[1].shape[1]
+                and getattr(self.mixer, "in_dtype", None) == getattr(self.feed_forward, "in_dtype", None)):
+            self._split = first[0].shape[0]
+            if (self._split * first[0].shape[1] * first[0].element_size()) % 16 == 0:          # (the second matrix starts as aligned as the first)
+                self.w_first = torch.cat(first, dim=0).contiguous()
+                self.mixer.use_input_weight(self.w_first[:self._split])
+                self.feed_forward.use_input_weight(self.w_first[self._split:])
+        self._readers = _Readers(self._parts()[1:], self._stacked)
 
     def _parts(self):
         return [self.mixer_norm, self.mixer] + ([self.feed_forward] if self.feed_forward is not None else [])
@@ -233,11 +260,19 @@ class ParallelBlock:
             rows = made.__getitem__
         last = self.feed_forward if self.feed_forward is not None else self.mixer
         then = norm_to_hand_on(next_reader, ctx.n_rows) if getattr(last, "hands_norm_on", False) else None
-        out = self.mixer.forward(rows(self.mixer), x, ctx, cache, then=then) if last is self.mixer and then is not None else self.mixer.forward(rows(self.mixer), x, ctx, cache)
+        own = [{}, {}]                            # what each half is told beyond its rows
+        w_first = self._stacked(ctx.n_rows)
+        if w_first is not None:
+            both = torch.empty((ctx.n_rows, w_first.shape[0]), dtype=torch.float32, device=x.device)
+            linear(rows(self.mixer), w_first, both)
+            own[0]["projected"], own[1]["projected"] = both[:, :self._split], both[:, self._split:]
+        if then is not None:
+            own[0 if last is self.mixer else 1]["then"] = then
+        out = self.mixer.forward(rows(self.mixer), x, ctx, cache, **own[0])
         if ctx.trace is not None:
             ctx.trace("attn_out", x)
         if self.feed_forward is not None:
-            out = self.feed_forward.forward(rows(self.feed_forward), x, ctx, then=then) if then is not None else self.feed_forward.forward(rows(self.feed_forward), x, ctx)
+            out = self.feed_forward.forward(rows(self.feed_forward), x, ctx, **own[1])
         if ctx.trace is not None:
             ctx.trace("ffn_out", x)
         return out if then is not None else None

@@ -56,6 +56,14 @@ class GatedDelta(Mixer):
     def weights_read_per_step(self):
         return [self.w_in, self.taps, self.a_log, self.dt_bias, self.out_norm, self.w_o]
 
+    # The first product's matrix, for a block that makes the first products of several parts in one (`ParallelBlock`): it then
+    # hands the part its rows of that product (`forward(..., projected=)`) and the part keeps a view of the common matrix.
+    def input_weight(self):
+        return self.w_in
+
+    def use_input_weight(self, view):
+        self.w_in = view
+
     @classmethod
     def tensor_needs(cls, spec):
         s, d = spec, spec.hidden_size
@@ -69,12 +77,14 @@ class GatedDelta(Mixer):
     def cache_need(cls, spec):
         return StateNeed((ops.delta_state_floats(spec.n_heads, spec.n_kv_heads, spec.key_dim, spec.value_dim, spec.conv_taps),), torch.float32)
 
-    def forward(self, h, residual, ctx, cache, then=None, overwrite=False):
+    def forward(self, h, residual, ctx, cache, then=None, overwrite=False, projected=None):
         s, T, o, dev = self.spec, ctx.n_rows, self.offsets, ctx.device
         H, G, dk, dv = s.n_heads, s.n_kv_heads, s.key_dim, s.value_dim
         vv = H * dv
-        proj = torch.empty((T, self.w_in.shape[0]), dtype=torch.float32, device=dev)
-        linear(h, self.w_in, proj)
+        proj = projected
+        if proj is None:
+            proj = torch.empty((T, self.w_in.shape[0]), dtype=torch.float32, device=dev)
+            linear(h, self.w_in, proj)
         seg_start, seg_len = ops.segments(ctx)
         qkv = torch.empty((T, 2 * G * dk + vv), dtype=torch.float32, device=dev)
         gates = torch.empty((T, 2 * H), dtype=torch.float32, device=dev)

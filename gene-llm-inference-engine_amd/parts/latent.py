@@ -86,6 +86,12 @@ class LatentAttention(Mixer):
     def weights_read_per_step(self):
         return [self.w_down, self.q_norm, self.kv_norm, self.w_uq, self.w_uk_t, self.w_uv, self.w_o]
 
+    def input_weight(self):          # (see `GatedDelta.input_weight`)
+        return self.w_down
+
+    def use_input_weight(self, view):
+        self.w_down = view
+
     @classmethod
     def tensor_needs(cls, spec):
         s, d = spec, spec.hidden_size
@@ -98,11 +104,13 @@ class LatentAttention(Mixer):
     def cache_need(cls, spec):
         return PagedKvNeed(1, spec.kv_rank + spec.rotary_dim, spec.window, spec.kv_rank, None)
 
-    def forward(self, h, residual, ctx, cache, then=None, overwrite=False):
+    def forward(self, h, residual, ctx, cache, then=None, overwrite=False, projected=None):
         s, T, dev = self.spec, ctx.n_rows, ctx.device
         H, kd = s.n_heads, self.key_dim
-        down = torch.empty((T, self.w_down.shape[0]), dtype=torch.float32, device=dev)
-        linear(h, self.w_down, down)
+        down = projected
+        if down is None:
+            down = torch.empty((T, self.w_down.shape[0]), dtype=torch.float32, device=dev)
+            linear(h, self.w_down, down)
         cos, sin = self.position.pair_tables(ctx) if self.position is not None else (None, None)
         cq = torch.empty((T, s.q_rank), dtype=self.cq_dtype, device=dev)
         ops.latent_prepare(down, s.q_rank, s.kv_rank, s.rotary_dim, self.q_norm, self.kv_norm, s.norm_eps, cos, sin, ctx.row_pos, ctx.row_slot,

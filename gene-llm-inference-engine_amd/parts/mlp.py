@@ -85,10 +85,18 @@ class DenseMlp(FeedForward):
         i, d = spec.intermediate_size, spec.hidden_size
         return [TensorNeed(spec.up_proj, (i, d)), TensorNeed(spec.down_proj, (d, i)), TensorNeed(spec.activation_params, (2,))]
 
-    def forward(self, h, residual, ctx, then=None, overwrite=False):
+    def input_weight(self):          # (the first product's matrix, for a block that makes several parts' first products in one)
+        return self.w_up
+
+    def use_input_weight(self, view):
+        self.w_up = view
+
+    def forward(self, h, residual, ctx, then=None, overwrite=False, projected=None):
         T, inter = ctx.n_rows, self.spec.intermediate_size
-        up = torch.empty((T, inter), dtype=torch.float32, device=ctx.device)
-        linear(h, self.w_up, up)
+        up = projected
+        if up is None:
+            up = torch.empty((T, inter), dtype=torch.float32, device=ctx.device)
+            linear(h, self.w_up, up)
         mid = torch.empty((T, inter), dtype=self.mid_dtype, device=ctx.device)
         ops.xielu(up, mid, self.params)
         if overwrite:
