@@ -123,6 +123,10 @@ class FeedForward(Part):
 #   takes_handed_norm(n_rows)      says that the part's first product can finish such a norm at this number of rows.
 #   hands_norm_on = True           `forward` takes a keyword `then`, the norm that will read `residual` next, adds onto the residual with
 #                                  `linear_onto(..., then)` and returns what that returns (the `HandedRows`, or None).
+#   input_weight()                 the matrix of the part's first product (its rows in the order the part reads the product's columns), or
+#                                  None; with it `use_input_weight(view)` (the same matrix as a view of a larger one, to keep instead of its
+#                                  own) and a keyword `projected` of `forward` (float32 [rows, that matrix's rows]: the product, already made).
+#                                  A block whose parts read the same rows may then make their first products as one (`ParallelBlock`).
 
 
 # Optional, for a block (an arrangement of parts; of however many halves):
