@@ -161,9 +161,9 @@ def rigalorn_beside_fekorax(args) -> int:
         fekorax = dict(architecture="Fekorax", vocab=vocab, width=D, embedding=dict(scale=D ** 0.5), norm=dict(eps=1e-5), layers=layers[:L], max_positions=T + 1024)
         delta = dict(type="delta", mlp=mlp, mixer=dict(heads=max(1, H // 4), kv_heads=max(1, H // 8), dim=hd, vdim=2 * hd, conv=4))
         latent = dict(type="latent_attention", mlp=mlp, mixer=dict(heads=H, dim=hd, rot_dim=hd // 2, vdim=hd, q_rank=12 * hd, kv_rank=4 * hd, scale=(1.5 * hd) ** -0.5,
-                                                                    rot=dict(dims=hd // 2, base=1e6), mask=dict(size=1024)))
+                                                                    rot=dict(dims=hd // 2, base=500000.0), mask=dict(size=1024)))
         blended = dict(type="attention", mlp=mlp, mixer=dict(heads=H, kv_heads=G, dim=hd, vdim=hd, scale=hd ** -0.5, v_mix=True, mask=dict(size=1024), rot=dict(
-            dims=hd // 2, base=10000.0, scaling=dict(factor=8.0, original=1024, fast=32.0, slow=1.0))))
+            dims=hd // 2, base=10000.0, scaling=dict(factor=4.0, original=4096, fast=16.0, slow=2.0))))
         rigalorn = dict(architecture="Rigalorn", vocab=vocab, width=D, embedding=dict(scale=D ** 0.5), norm=dict(eps=1e-5), max_positions=T + 1024,
                         layers=([delta, latent, blended, delta] * ((L + 3) // 4))[:L])
         record["sizes"][size] = {}

@@ -43,7 +43,7 @@ def test_stretched_frequencies_by_hand():
 
 def test_the_engine_s_configuration_computes_the_same_frequencies():
     from geneinfer_amd.config.rigalorn import YarnScaling, yarn_frequencies
-    for dims, base, s in ((8, 16.0, dict(factor=4.0, original=16, fast=2.0, slow=0.5)), (64, 10000.0, dict(factor=8.0, original=1024, fast=32.0, slow=1.0)),
+    for dims, base, s in ((8, 16.0, dict(factor=4.0, original=16, fast=2.0, slow=0.5)), (48, 20000.0, dict(factor=6.0, original=2048, fast=24.0, slow=2.0)),
                           (2, 7.0, dict(factor=2.0, original=8, fast=1.0, slow=1.0)), (16, 100.0, dict(factor=3.0, original=4096, fast=0.001, slow=0.0005))):
         scaling = YarnScaling(s["factor"], s["original"], s["fast"], s["slow"])
         f, mag = P.rotary_frequencies(dims, base, s)
