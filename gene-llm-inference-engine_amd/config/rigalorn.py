@@ -53,9 +53,10 @@ class YarnScaling:
 
 
 def yarn_frequencies(dims: int, base: float, scaling: YarnScaling):
-    """The dims/2 frequencies: f_i = base^(-2i/dims), blended as f_i / factor * ramp_i + f_i * (1 - ramp_i), where ramp_i climbs
-    from 0 at index lo to 1 at index hi and index(t) = dims * ln(original / (2 pi t)) / (2 ln base) is the (fractional) pair that
-    makes t turns over the original context."""
+    """The dims/2 frequencies.  Pair i turns at base^(-2i/dims); the pair that makes exactly t turns over the original context is the
+    (fractional) one at index(t) = dims ln(original / (2 pi t)) / (2 ln base).  Pairs up to lo = floor(index(fast)) keep their
+    frequency, pairs from hi = ceil(index(slow)) on turn `factor` times slower, and between the two the share r_i of the slow
+    frequency climbs linearly from 0 to 1: f_i (1 - r_i) + (f_i / factor) r_i."""
     index = lambda turns: dims * math.log(scaling.original / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
     lo = max(math.floor(index(scaling.fast)), 0)
     hi = min(math.ceil(index(scaling.slow)), dims - 1)

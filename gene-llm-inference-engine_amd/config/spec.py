@@ -154,7 +154,7 @@ class SwiGluSpec:
 @dataclass(frozen=True)
 class DenseMlpSpec:
     """down(act(up(x))), no gate, no biases.  `activation` "xielu": with the two numbers (p, q) of the tensor `activation_params`,
-    act(z) = softplus(p) z^2 + z/2 for z > 0 and (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2 otherwise."""
+    and a = softplus(p), b = 1/2 + softplus(q): act(z) = z/2 + a z^2 on the right of zero and z/2 + b (e^z - 1 - z) on the left."""
     kind: ClassVar[str] = "dense_mlp"
     hidden_size: int
     intermediate_size: int
@@ -166,12 +166,13 @@ class DenseMlpSpec:
 
 @dataclass(frozen=True)
 class GatedDeltaSpec:
-    """The gated delta rule: per head a memory S [key_dim, value_dim], zero at a sequence's start, and per token
-        S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q
-    with g = exp(-exp(a_log) softplus(a(x) + dt_bias)) and beta = sigmoid(b(x)) per head.  q and k (n_kv_heads heads, head h of
+    """The gated delta rule: per head a memory M [key_dim, value_dim], zero at a sequence's start.  A token first lets it decay,
+    M <- d M; then corrects what it holds along the token's key towards the token's value, M <- M + k e^T with e = s (v - M^T k);
+    then reads it with the query, y = M^T q (so the read-out sees the token's own correction).  Per head the decay is
+    d = exp(-exp(a_log) softplus(a(x) + dt_bias)) and the step size s = sigmoid(b(x)).  q and k (n_kv_heads heads, head h of
     the memory uses q/k head h // (n_heads / n_kv_heads)) and v pass a causal convolution of `conv_taps` taps per channel
     (tensors [channels, taps], the last tap the token's own) and SiLU; q and k are then divided by sqrt(sum of squares + 1e-6),
-    q also by sqrt(key_dim).  Every head's o is divided by its root mean square (`norm_eps`), multiplied by `out_norm`
+    q also by sqrt(key_dim).  Every head's y is divided by its root mean square (`norm_eps`), multiplied by `out_norm`
     [value_dim], one for all heads, and by SiLU(gate(x)), and goes through `o_proj`."""
     kind: ClassVar[str] = "gated_delta"
     hidden_size: int

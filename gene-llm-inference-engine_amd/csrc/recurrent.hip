@@ -22,10 +22,9 @@
 // are then taken for all 64 at once.  Every sum's order is fixed by dk alone: a request's results have the same bits however
 // its rows are cut into steps.
 //
-// The gated delta rule keeps a memory S [dk][dv] per head and, per token with decay g, step size beta, unit key k, query q:
-//     S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q
-// (what the memory holds along k is moved towards v, then read with q: the read-out sees the token's own write).  Columns of S
-// never meet here either, so a wave owns four of them, lanes as above; a token costs two sums over the key's rows instead of
+// The gated delta rule keeps a memory M [dk][dv] per head.  A token with decay d, step size s, unit key k and query q lets it decay,
+// M <- d M, moves what it holds along k towards v, M <- M + k e^T with e = s (v - M^T k), and reads it, y = M^T q: the read-out
+// sees the token's own write.  Columns of M never meet here either, so a wave owns four of them, lanes as above; a token costs two sums over the key's rows instead of
 // one, the second of which waits for the first.  Before the rule, q, k and v pass a short causal convolution over the
 // request's rows (the last taps - 1 rows before a step are part of the request's state) and SiLU, and q and k are made unit
 // vectors; after it, a head's output is divided by its root mean square, as the matrix memory's.
@@ -317,11 +316,11 @@ __global__ __launch_bounds__(256) void delta_tail_kernel(const float* __restrict
     }
 }
 
-// The rule itself: one wave per (request of the step, head, four columns of S).  lane = column * 16 + group of rows; a lane keeps
+// The rule itself: one wave per (request of the step, head, four columns of M).  lane = column * 16 + group of rows; a lane keeps
 // the rows 16 apart of its column.  State of a request slot: [head][tile]{[dk][4]}.
-// With S the memory before the token, S' = g S + k w^T after it and w = beta (v - g S^T k), the read-out is
-//     o = S'^T q = g S^T q + w (k . q):
-// both sums over the old memory's rows (S^T k and S^T q) and k . q are taken in one pass and reduced side by side, the memory is
+// With M the memory before the token, M' = d M + k e^T after it and e = s (v - d M^T k), the read-out is
+//     y = M'^T q = d M^T q + e (k . q):
+// both sums over the old memory's rows (M^T k and M^T q) and k . q are taken in one pass and reduced side by side, the memory is
 // updated behind them, and a token's chain of dependent steps is one pass and one reduction, not two of each.  Every sum over the
 // key's rows is the lanes' own shares in a fixed order, then the 16 groups by lane moves: the bits do not depend on the cut.
 // Key and query of a block of tokens wait in LDS; the block after it is asked for while this one is worked on.
@@ -402,7 +401,7 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict_
             sk = group_sum<RG>(sk);
             sq = group_sum<RG>(sq);
             kq = group_sum<RG>(kq);
-            const float w = gb.y * (v_s[buf][u][c] - gb.x * sk);       // beta (v - g S^T k)
+            const float w = gb.y * (v_s[buf][u][c] - gb.x * sk);       // s (v - d M^T k)
 #pragma unroll
             for (int rr = 0; rr < ROWS; ++rr) S[rr] = fmaf(gb.x, S[rr], kx[rr] * w);
             if (rg == 0 && live) out[(size_t)(t0 + b0 + u) * ldo + h * dv + col] = fmaf(gb.x, sq, w * kq);

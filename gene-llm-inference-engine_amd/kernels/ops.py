@@ -727,7 +727,7 @@ def delta_tail(proj, conv_off, n_taps, seg_start, seg_len, row_slot, state, n_he
 
 def delta_scan(qkv, gates, seg_start, seg_len, row_slot, state, out, n_heads, n_kv, dk, dv):
     """The gated delta rule over every request's rows of the step, in order (csrc/recurrent.hip states it): qkv and gates as
-    `delta_prepare` leaves them, out float32 [n, heads*dv] gets the read-outs S^T q; the memories come from the request's state
+    `delta_prepare` leaves them, out float32 [n, heads*dv] gets the read-outs M^T q; the memories come from the request's state
     slot and go back into it."""
     _dev(qkv, gates, seg_start, seg_len, row_slot, state, out)
     n = qkv.shape[0]

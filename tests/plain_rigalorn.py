@@ -31,7 +31,7 @@ def softplus(z):
 
 
 def xielu(z, p, q):
-    """z > 0: softplus(p) z^2 + z/2;  z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2."""
+    """With a = softplus(p) and b = 1/2 + softplus(q): z/2 + a z^2 on the right of zero, z/2 + b (e^z - 1 - z) on the left."""
     right = softplus(p) * z * z + z / 2
     left = (0.5 + softplus(q)) * (torch.expm1(torch.clamp(z, max=0)) - z) + z / 2
     return torch.where(z > 0, right, left)
@@ -159,8 +159,8 @@ def short_conv_silu(x, taps):
 
 
 def delta_rule(q, k, v, beta, g):
-    """One head.  q, k [T, dk], v [T, dv], beta, g [T].  S starts at zero; per token: S <- g S; u = beta (v - S^T k);
-    S <- S + k u^T; o = S^T q."""
+    """One head.  q, k [T, dk], v [T, dv], beta (step sizes), g (decays) [T].  The memory starts at zero; a token lets it decay, moves
+    what it holds along the token's key towards the token's value by the step size, and is read with the query."""
     S = q.new_zeros(q.shape[1], v.shape[1])
     out = []
     for t in range(q.shape[0]):
