@@ -24,10 +24,11 @@
 //
 // The gated delta rule keeps a memory M [dk][dv] per head.  A token with decay d, step size s, unit key k and query q lets it decay,
 // M <- d M, moves what it holds along k towards v, M <- M + k e^T with e = s (v - M^T k), and reads it, y = M^T q: the read-out
-// sees the token's own write.  Columns of M never meet here either, so a wave owns four of them, lanes as above; a token costs two sums over the key's rows instead of
-// one, the second of which waits for the first.  Before the rule, q, k and v pass a short causal convolution over the
-// request's rows (the last taps - 1 rows before a step are part of the request's state) and SiLU, and q and k are made unit
-// vectors; after it, a head's output is divided by its root mean square, as the matrix memory's.
+// sees the token's own write.  Columns of M never meet here either, so a wave owns four of them, lanes as above; a token costs
+// two sums over the key's rows, which the kernel takes in one pass over the memory as it was before the token.  Before the rule,
+// q, k and v pass a short causal convolution over the request's rows (the last taps - 1 rows before a step are part of the
+// request's state) and SiLU, and q and k are made unit vectors; after it, a head's output is divided by its root mean square, as
+// the matrix memory's.
 #include "common.h"
 
 namespace {
